@@ -1,9 +1,12 @@
 /* C ABI of librwkv7_mi355x.so: the RWKV7 generalized delta rule on MI355X (gfx950).
  *
- * Plain pointers and sizes only; every pointer is DEVICE memory owned by the caller.
- * The library never allocates, never synchronises and keeps no mutable global
- * state; every call enqueues its kernels on the hipStream_t passed as `stream`
- * (NULL = the default stream) on the caller's current device and returns.
+ * Plain pointers and sizes only; every pointer is DEVICE memory owned by the caller
+ * unless a comment says otherwise.  The library never allocates and never
+ * synchronises; every call enqueues its kernels on the hipStream_t passed as `stream`
+ * (NULL = the default stream) on the caller's current device and returns.  The only
+ * state it keeps between calls is a process-wide launch counter (an atomic), from
+ * which every chunked forward launch draws a fresh 64-bit tag; calls from several
+ * threads are safe.
  *
  * Return value of every int function: 0 = ok, < 0 = argument error (RWKV7_ERR_*,
  * nothing was launched), > 0 = a hipError_t reported by a launch.
@@ -92,6 +95,32 @@ int rwkv7_fwd(const void* r, const void* w, const void* k, const void* v,
               int B, int T, int H, int K, int V, int dtype,
               void* ws, size_t ws_bytes, void* stream);
 
+/* ---- did a chunked forward finish? ------------------------------------------------
+ * The one-kernel chunked forward hands each (batch, head) state from one 64-token
+ * chunk's workgroup to the next through the workspace; a workgroup waits for its
+ * predecessor for at most two seconds (a chunk takes microseconds).  Should a wait
+ * ever time out -- which no correct launch does -- the kernel still drains: the
+ * waiting waves stop, fill what they would have written of o and ht with NaN, and
+ * leave a mark in a 16-byte status record inside the workspace.  The call itself has
+ * returned 0 long before, so this record is how a caller tells "the library gave
+ * up" from "my inputs held NaN": after synchronising the stream ITSELF, copy the 16
+ * bytes at  (char*)ws + rwkv7_fwd_status_offset(B, T, H, dtype)  to the host and
+ * pass them to rwkv7_fwd_status().  The record belongs to the last forward that ran
+ * with this workspace: rwkv7_fwd and rwkv7_fwd_gather (offset from
+ * rwkv7_fwd_status_offset), rwkv7_fwd_varlen (rwkv7_fwd_varlen_status_offset), and the
+ * two-kernel form, whose summary launch writes a record that can only read "done".
+ * The offset functions return RWKV7_NO_STATUS_RECORD for shapes and dtypes whose call
+ * runs no chunked kernel (T <= 12, float32, float16; K = V = 128).  No counterpart in the reference,
+ * whose kernels do not communicate. */
+#define RWKV7_NO_STATUS_RECORD ((size_t)-1)
+#define RWKV7_FWD_DONE      0   /* the launch that wrote the record did not give up */
+#define RWKV7_FWD_GAVE_UP   1   /* a hand-off wait timed out: o and ht hold NaN */
+#define RWKV7_FWD_NO_LAUNCH 2   /* the record is zero: no launch has written it */
+size_t rwkv7_fwd_status_offset(int B, int T, int H, int dtype);
+size_t rwkv7_fwd_varlen_status_offset(int n_seq, int T_total, int H, int dtype);
+/* `record`: HOST pointer to a copy of the 16-byte record.  Returns RWKV7_FWD_* or RWKV7_ERR_NULL_POINTER. */
+int rwkv7_fwd_status(const void* record);
+
 /* ---- initial states gathered through a map -----------------------------------------
  * The reference's RWKV6 operator lets several batch rows start from one of a few
  * stored states: init_state [n_state, H, K, K] with state_map [B]
@@ -123,8 +152,8 @@ int rwkv7_decode_step_gather(const void* r, const void* w, const void* k, const 
  * (torch_op.py:81-98: cumsum, intra-chunk A, WY inverse, w/u) and fills ws;
  * rwkv7_fwd_chunk_scan replaces its serial scan and output launches
  * (torch_op.py:101-117) and consumes ws.  bf16 only (f32: RWKV7_ERR_UNSUPPORTED);
- * the same ws (rwkv7_fwd_chunk_workspace_bytes, 32.25 KiB per chunk and head) must be
- * passed to both. */
+ * the same ws (rwkv7_fwd_chunk_workspace_bytes, 32.25 KiB per chunk and head, + 256 bytes
+ * for the status record at offset rwkv7_fwd_chunk_workspace_bytes() - 256) must be passed to both. */
 size_t rwkv7_fwd_chunk_workspace_bytes(int B, int T, int H, int dtype);
 int rwkv7_fwd_chunk_summary(const void* r, const void* w, const void* k, const void* v,
                             const void* a, const void* b,
@@ -162,8 +191,9 @@ int rwkv7_bwd(const void* r, const void* w, const void* k, const void* v,
  * stripped, e.g. triton_kernel/chunk_h_fwd.py:51-58).  These calls implement that
  * meaning: r..b, o and the gradients are [T_total, H, 64]; cu_seqlens is int32
  * [n_seq + 1] on the device, starting at 0, non-decreasing, ending at T_total at most
- * (tokens beyond the last entry are left alone; values are clamped into [0, T_total]
- * on the device, so a bad table gives meaningless results, never a fault); h0, ht, d_ht
+ * (rows of o and of the gradients beyond the last entry are filled with zeros; values are
+ * clamped into [0, T_total] on the device and a table whose spans overlap has the chunks
+ * beyond T_total / 64 + n_seq dropped, so a bad table gives meaningless results, never a fault); h0, ht, d_ht
  * and dh0 are float32 [n_seq, H, 64, 64] (h0_batch_stride 0 broadcasts one state).  A
  * sequence may be empty: its final state is its initial state.  Chunks are counted from
  * each sequence's own first token, so the result for a sequence does not depend on

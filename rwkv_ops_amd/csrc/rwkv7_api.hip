@@ -1,5 +1,5 @@
 // extern "C" entry points of librwkv7_mi355x.so: argument validation, then launch.
-// Nothing here allocates, synchronises or keeps state between calls.
+// Nothing here allocates or synchronises.
 #include "../../include/rwkv7_mi355x.h"
 #include "../../include/rwkv6_mi355x.h"
 #include "rwkv7_kernels.h"
@@ -108,6 +108,19 @@ size_t rwkv7_fwd_workspace_bytes(int B, int T, int H, int dtype) {
     if (dtype != RWKV7_DTYPE_BF16 || B < 1 || T < 2 || H < 1) return 0;
     return use_fused_forward(B, H) ? rwkv7::fwd_fused_workspace_bytes(B, T, H)
                                    : rwkv7::fwd_chunk_workspace_bytes(B, T, H);
+}
+
+size_t rwkv7_fwd_status_offset(int B, int T, int H, int dtype) {
+    if (dtype != RWKV7_DTYPE_BF16 || B < 1 || T <= RECURRENT_MAX_T || H < 1) return RWKV7_NO_STATUS_RECORD;
+    return use_fused_forward(B, H) ? rwkv7::fwd_fused_status_offset(B, T, H)
+                                   : rwkv7::fwd_chunk_status_offset(B, T, H);
+}
+
+int rwkv7_fwd_status(const void* record) {
+    if (!record) return RWKV7_ERR_NULL_POINTER;
+    const unsigned long long* rec = static_cast<const unsigned long long*>(record);
+    if (rec[1] == 0ull) return RWKV7_FWD_NO_LAUNCH;
+    return rec[0] == rec[1] ? RWKV7_FWD_GAVE_UP : RWKV7_FWD_DONE;
 }
 
 size_t rwkv7_fwd_chunk_workspace_bytes(int B, int T, int H, int dtype) {
@@ -238,6 +251,12 @@ size_t rwkv7_fwd_varlen_workspace_bytes(int n_seq, int T_total, int H, int dtype
     if (dtype != RWKV7_DTYPE_BF16 || n_seq < 1 || T_total < 1 || H < 1) return 0;
     return use_fused_forward(n_seq, H) ? rwkv7::fwd_fused_workspace_bytes(n_seq, T_total, H, true)
                                        : rwkv7::fwd_chunk_workspace_bytes(n_seq, T_total, H, true);
+}
+
+size_t rwkv7_fwd_varlen_status_offset(int n_seq, int T_total, int H, int dtype) {
+    if (dtype != RWKV7_DTYPE_BF16 || n_seq < 1 || T_total < 1 || H < 1) return RWKV7_NO_STATUS_RECORD;
+    return use_fused_forward(n_seq, H) ? rwkv7::fwd_fused_status_offset(n_seq, T_total, H, true)
+                                       : rwkv7::fwd_chunk_status_offset(n_seq, T_total, H, true);
 }
 
 int rwkv7_fwd_varlen(const void* r, const void* w, const void* k, const void* v, const void* a,

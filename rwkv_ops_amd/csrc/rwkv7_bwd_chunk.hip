@@ -45,14 +45,6 @@
 
 namespace rwkv7 {
 
-#ifdef RWKV7_DEBUG
-__device__ unsigned long long* g_ts = nullptr;
-extern "C" int rwkv7_debug_set_ts(void* p) { return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_ts), &p, sizeof(p)); }
-#define DBG_T(i) do { if (g_ts && n == 2000 && threadIdx.x == 0) g_ts[i] = wall_clock64(); } while (0)
-#else
-#define DBG_T(i) do { } while (0)
-#endif
-
 namespace {
 
 // Log decays are kept in base 2 (as in rwkv7_fwd_chunk.hip), so every exponential is one v_exp_f32.
@@ -291,7 +283,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     const int ch0 = 32 * hf + 8 * g;          // first of this lane's eight channels in the load layout
     const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 
-    DBG_T(0);
     auto prefetch_next = [&](auto part) {
         if (n_next >= 0)
             load_chunk_inputs<decltype(part)::value, PACKED>(next, n_next, lane, r_, w_, k_, v_, a_, b_, dO_, hs, dhs, L);
@@ -318,7 +309,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         gstep[e] = valid ? fmaxf(-LOG2E * ex2(LOG2E * wv), G_MIN2) : 0.f;     // log2 of exp(-exp(w))
         gl[e] = row_inclusive_scan(gstep[e]);
     }
-    DBG_T(13);
     float* tot = reinterpret_cast<float*>(smem + OFF_TOT);
     if (x == 15) {
         float4_t* dst = reinterpret_cast<float4_t*>(tot + w * 64 + ch0);
@@ -326,7 +316,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         dst[1] = float4_t{gl[4], gl[5], gl[6], gl[7]};
     }
     __syncthreads();
-    DBG_T(14);
     float xmax = 0.f;
     {
         float pre[8], gother[8];               // gother: chunk totals of the other half's channels (for npass)
@@ -406,7 +395,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     {
         bf16x8_t Qp, Ap, Kp, Bp;
         bucket_operands(0, R, K, A, B, Qp, Ap, Kp, Bp);
-        DBG_T(15);
         put_operands(Qp, Ap, Kp, Bp);
         put_row(S_V, V); put_row(S_DO, DO);
 #pragma unroll
@@ -418,7 +406,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     }
     __syncthreads();
 
-    DBG_T(1);
     // ---- G1: block row w (rows j, column i = 16w + x) of Aqk, Aqb (waves hf = 0) and of Aak, Aab
     // (waves hf = 1), bucket by bucket
     float4_t acc1[4], acc2[4];
@@ -475,7 +462,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         tile_store_acc(smem, hf ? S_AAK : S_AQK, w, J, lane, J <= w ? acc1[J] : zero4);
         tile_store_acc(smem, hf ? S_AAB : S_AQB, w, J, lane, J <= w ? acc2[J] : zero4);
     }
-    DBG_T(2);
     // ---- inverse of the diagonal block (see chunk_summary_kernel); the waves that hold Aab do it
     float4_t Dm = zero4;
     if (hf) {
@@ -527,7 +513,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     }
     __syncthreads();                       // Aab is dead from here: its slot takes h0
 
-    DBG_T(3);
     // ---- h0^T tile [v][c] from the float image; wave = (value tile w, key tiles 2hf, 2hf + 1)
 #pragma unroll
     for (int m = 0; m < 2; ++m) tile_store_acc(smem, S_H0, w, 2 * hf + m, lane, h0img[m]);
@@ -578,7 +563,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     };
 
     float4_t tmp[2];
-    DBG_T(4);
     // Y[j][v] = ag h0 + Aak V        -> Y^T[v][j]
     clear(tmp);
     gemm(tmp, rowsA(S_AG), rowsB(S_H0));
@@ -591,7 +575,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     store_tile(S_SA, tmp);
     __syncthreads();                       // Y is dead: its slot takes dh'
 
-    DBG_T(5);
     // ---- dh'^T tile [v][c]; the decay part of dG needs  sum_v h0 dh'  in float32
     {
         float dgdec[8];                    // partial over this lane's value column, key rows 16(2hf+m)+4g+e
@@ -615,7 +598,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     put_row(S_BG, BG);
     __syncthreads();
 
-    DBG_T(6);
     // accumulators that live to the end: rows = tokens, column = channel 16w + x
     float4_t acc_q[2], acc_a[2], acc_kg[2], acc_bg[2], acc_v[2];
     clear(acc_q); clear(acc_a); clear(acc_kg); clear(acc_bg); clear(acc_v);
@@ -639,7 +621,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     gemm_ar(acc_v, colsA(S_AQK), DOc);
     gemm_ar(acc_v, rowsA(S_KG), DHr);
     __syncthreads();                       // dh' is dead: its slot takes dY
-    DBG_T(7);
     // dY[j][v] = M^T dSA              -> dY^T[v][j]
     clear(tmp);
     gemm(tmp, rowsA(S_MT), rowsB(S_DSA));
@@ -649,7 +630,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     gemm(acc_a, colsA(S_DY), colsB(S_H0));         // dag_h[i][c] = dY h0^T
     __syncthreads();                       // h0 is dead: its slot takes dAqk
 
-    DBG_T(8);
     prefetch_next(P1{});   // the next chunk's inputs land while the last products and the epilogue run
     // ---- dA matrices as tiles [i][j] (column tile w = token tile i; rows of the product are j).  Their
     // slots (h0, M^T, kg, dSA) are dead since the last barrier, so each is stored as soon as it is masked.
@@ -677,7 +657,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     }
     __syncthreads();
 
-    DBG_T(9);
     prefetch_next(P2{});
     // ---- the decay-weighted products and the epilogue in the load layout.
     // dgi / dge are formed from the SAME bf16-rounded operands the products used (z qg - z kt - ...), not
@@ -723,22 +702,18 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         }
         // this lane's pieces of the bucket-0 operands, back from their tiles
         const bf16x8_t Qp = get_row(S_QG), Ap = get_row(S_AG), Kp = get_row(S_KT), Bp = get_row(S_BT);
-        DBG_T(10);
         prefetch_next(P3{});
         // Every tile is dead now, so all seven accumulator sets change layout in one round: float
         // tiles [channel][token] over the whole tile area, one barrier before and one after.
         __syncthreads();
-        DBG_T(16);
         auto stg = [&](int i) { return reinterpret_cast<float*>(smem + i * (64 * LDZ * 4)); };
         stage_put(stg(0), acc_k); stage_put(stg(1), acc_kg); stage_put(stg(2), acc_v);
         stage_put(stg(3), acc_b); stage_put(stg(4), acc_bg); stage_put(stg(5), acc_q); stage_put(stg(6), acc_a);
         __syncthreads();
-        DBG_T(17);
         float zk[8], zkg[8], zv[8], zb[8], zbg[8], zq[8], za[8];
         stage_get(stg(0), zk); stage_get(stg(1), zkg); stage_get(stg(2), zv);
         stage_get(stg(3), zb); stage_get(stg(4), zbg); stage_get(stg(5), zq); stage_get(stg(6), za);
         float out[8];
-        DBG_T(18);
         prefetch_next(P4{});
         float ek[8], et[8];
 #pragma unroll
@@ -771,7 +746,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
             sall[e] += dge[e] - dkk[e];
         }
         store_rows(da_, pack_rows(out));
-        DBG_T(19);
     } else {
         // Several decay buckets (strong decays): one pass of the products per bucket, each with its own
         // exponent offset, accumulated in registers.
@@ -862,7 +836,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
 #pragma unroll
         for (int e = 0; e < 8; ++e) sall[e] = dgi[e] - dkk[e] + dge[e];
     }
-    DBG_T(11);
     // dG = e^G sum_v(h0 dh') + sum over the 64 tokens of dkk;  dg = suffix_sum(dgi + dge) - dge + dG
     float dg[8];
     {
@@ -911,7 +884,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         for (int e = 0; e < 8; ++e) dwv[e] = dg[e] * (LN2 * gstep[e]);     // d/dw of g = -exp(w) is g itself
         store_rows(dw_, pack_rows(dwv));
     }
-    DBG_T(12);
 }
 
 #define RWKV7_BWD_PARAMS \

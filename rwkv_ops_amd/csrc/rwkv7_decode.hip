@@ -25,11 +25,6 @@
 
 namespace rwkv7 {
 
-#ifdef RWKV7_DEBUG
-int g_decode_variant = 0;
-extern "C" void rwkv7_debug_decode_variant(int v) { g_decode_variant = v; }
-#endif
-
 constexpr int DECODE_WAVES = 4;   // half-heads per workgroup
 
 __device__ __forceinline__ float reduce_ks(float x) { return sum_lane_groups_of_8(x); }
@@ -124,18 +119,6 @@ static hipError_t launch_decode_t(const SeqArgs& p, hipStream_t stream) {
             p.ht_in_place ? 1 : 0, p.B, p.H);
         return hipGetLastError();
     }
-#ifdef RWKV7_DEBUG
-    extern int g_decode_variant;
-    auto args = [&](auto kern) {
-        kern<<<dim3(grid), dim3(64 * DECODE_WAVES), 0, stream>>>(
-            (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, (const T*)p.a, (const T*)p.b,
-            p.h0, p.h0_batch_stride, p.h0_map, p.n_state, (T*)p.o, p.ht_in_place ? const_cast<float*>(p.h0) : p.ht,
-            p.ht_in_place ? 1 : 0, p.B, p.H);
-    };
-    if (g_decode_variant == 1) { args(decode_kernel<T, false, false>); return hipGetLastError(); }
-    if (g_decode_variant == 2) { args(decode_kernel<T, true, false>); return hipGetLastError(); }
-    if (g_decode_variant == 3) { args(decode_kernel<T, false, true>); return hipGetLastError(); }
-#endif
     if (p.u6 != nullptr) {
         decode_kernel<T, true, true, true><<<dim3(grid), dim3(64 * DECODE_WAVES), 0, stream>>>(
             (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, nullptr, (const T*)p.u6,

@@ -86,10 +86,6 @@ __device__ __forceinline__ bf16x8_t load_frag_global(const bf16_t* p, bool valid
     return *reinterpret_cast<const bf16x8_t*>(p);
 }
 
-#ifdef RWKV7_DEBUG
-__device__ unsigned char* g_dbg = nullptr;
-#endif
-
 // Device-scope ("sc1") 16-byte accesses for the state hand-off of the fused kernel: four 16-byte
 // pieces 1 KiB apart per lane (the four key tiles of one value tile of a state image).  They bypass
 // the per-XCD L2, so a workgroup on any XCD sees what another one wrote once the writer's
@@ -116,19 +112,6 @@ __device__ __forceinline__ void state_load_agent_wait(float4_t (&h)[4]) {
 
 }  // namespace
 
-#ifdef RWKV7_DEBUG
-__device__ unsigned long long* g_fts = nullptr;
-extern "C" int rwkv7_debug_set_fts(void* p) { return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_fts), &p, sizeof(p)); }
-#define FTS(i) do { if (g_fts && bh == 5 && threadIdx.x == 0) g_fts[c * 16 + (i)] = wall_clock64(); } while (0)
-#else
-#define FTS(i) do { } while (0)
-#endif
-#ifdef RWKV7_DEBUG
-extern "C" int rwkv7_debug_set_dump(void* p) {
-    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_dbg), &p, sizeof(p));
-}
-#endif
-
 // Workspace arrays, all indexed by chunk id n = c * (B * H) + (b * H + h): the heads of one chunk
 // position are adjacent, so that concurrently running workgroups / scan waves touch one contiguous
 // region (and neighbouring 128-byte pieces of the same input rows) instead of 2^k-strided ones:
@@ -147,6 +130,9 @@ extern "C" int rwkv7_debug_set_dump(void* p) {
 // itself, taking the state from the workgroup of the previous chunk of the same head and handing its
 // own to the next one (see the end of the kernel).
 constexpr int MODE_FWD = 0, MODE_BWD = 1, MODE_FUSED = 2;
+// how long a fused workgroup waits for its predecessor's state before it gives up: two seconds of the
+// 100 MHz constant-rate clock (a chunk takes microseconds)
+constexpr unsigned long long WAIT_LIMIT_TICKS = 200000000ull;
 
 struct FusedArgs {
     const bf16_t* u;           // V6 only: the bonus vector [H][64]
@@ -158,8 +144,9 @@ struct FusedArgs {
     bf16_t* o;
     float* ht;                 // nullable
     float* hbuf;               // [2][B*H][4 value tiles][4 key tiles][64 lanes][4] float hand-off slots
-    unsigned long long* cnt;   // [B*H][4] tag + chunks completed per (head, value tile), then one give-up flag
+    unsigned long long* cnt;   // [B*H][4] tag + chunks completed per (head, value tile)
     unsigned long long tag;    // this launch's random 64-bit tag: the counters need no clearing (see launch_fwd_fused)
+    unsigned long long* status; // nullable: [0] = give-up flag (== tag: a hand-off wait timed out), [1] = tag of the launch
 };
 
 // V6 = true turns the kernel into the RWKV6 operator (/root/reference/rwkv_ops/rwkv6_kernel/
@@ -182,6 +169,12 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
     const int x = lane & 15, g = lane >> 4;
     // (Consecutive workgroups go to consecutive XCDs.  Giving each XCD a contiguous block of heads instead
     // of every eighth one was tried: + 1 % at 256 sequences, but twice as slow at 128.)
+    // The first workgroup (dispatched first) opens the launch's status record: "not given up", then the tag.
+    // A replay of a captured graph repeats the tag, so the flag an earlier replay may have left is taken away here.
+    if (blockIdx.x == 0 && threadIdx.x == 0 && fa.status != nullptr) {
+        __hip_atomic_store(fa.status, fa.tag - 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(fa.status + 1, fa.tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
     const ChunkCoord cc = chunk_coord(L, (int)blockIdx.x);
     if (!cc.live) return;              // packed sequences: the grid covers the most chunks there can be
     const int H = L.H, BH = L.B * L.H;
@@ -192,7 +185,6 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
     const bool valid = t < T;
     const int64_t row = ((cc.tok0 + t) * H + hi) * HEAD;
 
-    FTS(0);
     // ---- P0: load the chunk.  Lane (x, g) takes channels 8g..8g+7 and 32+8g..32+8g+7 of token x:
     // exactly the "plain" MFMA fragments of k-steps 0 and 1 for this wave's 16-token tile.
     bf16x8_t R[2], K[2], V[2], A[2], B[2];
@@ -239,7 +231,6 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         }
     }
     __syncthreads();                                                           // B0
-    FTS(5);
     float gsum[16];                    // chunk total per channel (<= 0)
     {
         // totals of the four waves; the prefix of waves before this one is picked by a wave-uniform
@@ -337,7 +328,6 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         *reinterpret_cast<bf16x8_t*>(smem + OFF_V + (t_local * LDT + col) * 2) = V[s];
     }
     __syncthreads();                                                           // B1
-    FTS(6);
     bf16x8_t DOr[2];                   // MODE_BWD: this lane's row of dO, on its way to the tile V leaves at B3
     if constexpr (BWD) {
         if (fa.d_o != nullptr && valid) {
@@ -441,7 +431,6 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         }
     }
     __syncthreads();                                                           // B2
-    FTS(7);
 
     // ---- P3: T1 = Aak V for this wave's 16 value columns (kept in registers), and the inverse of
     // the diagonal block: (I - N)^-1 = (I + N)(I + N^2)(I + N^4)(I + N^8), N strictly lower 16x16.
@@ -476,7 +465,6 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
     // DmT lane (column i' = x, rows j' = 4g..): DmT[j'][i'] = Dinv[i'][j'] -> row i' of Dinv, columns 4g..4g+3
     if constexpr (!V6) *reinterpret_cast<bf16x4_t*>(smem + OFF_DI + w * 512 + (x * 16 + 4 * g) * 2) = pack4(DmT);
     __syncthreads();                                                           // B3 (all T1 reads of Aak done)
-    FTS(8);
     if constexpr (BWD) {               // V is in registers (Vtr) everywhere: its tile takes dO
 #pragma unroll
         for (int s = 0; s < 2; ++s)
@@ -515,12 +503,6 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
             Xu[I] = pack4(uacc[I]);
         }
     }
-    FTS(9);
-#ifdef RWKV7_DEBUG
-    __syncthreads();
-    if (g_dbg && blockIdx.x == 0) { for (int i = threadIdx.x; i < LDS_BYTES; i += 256) g_dbg[i] = smem[i]; }
-    __syncthreads();
-#endif
     const bool single = npass == 1;
     if constexpr (BWD) { if (single) __syncthreads(); }        // the dO tile is complete (several buckets: B4)
     if (!single) {
@@ -534,7 +516,6 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         }
         __syncthreads();                                                       // B5
     }
-    FTS(10);
 
     // ---- P5: the register-resident chains for key-channel tile w (W) and value tile w (U)
     const bf16x8_t Ws[2] = {pack_sigma(wacc[0], wacc[1]), pack_sigma(wacc[2], wacc[3])};
@@ -632,7 +613,6 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
     if (single) end_of_chunk_products(std::true_type{}); else end_of_chunk_products(std::false_type{});
 
     if constexpr (MODE == MODE_FUSED) {
-        FTS(1);
         // ---- apply the chunk to the state.  State at the start of the chunk: chunk 0 takes h0, later
         // chunks wait for the previous chunk's workgroup (lower block index, hence already dispatched)
         // to publish value tile w.  Data and counter are device-scope accesses; the producer's
@@ -655,20 +635,24 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         } else {
             unsigned long long* cnt = fa.cnt + bh * 4 + w;
             if (lane == 0) {
-                // The previous chunk's wave w publishes exactly tag + c.  Bounded wait: after about a second
-                // without progress (or as soon as any other wave has given up) the wave stops waiting and
-                // poisons its outputs, so the grid always drains.
+                // The previous chunk's wave w publishes exactly tag + c.  Bounded wait: after WAIT_LIMIT_TICKS of
+                // the constant-rate clock without progress (or as soon as any other wave has given up) the wave
+                // stops waiting and poisons its outputs, so the grid always drains.  The clock and the shared
+                // flag are looked at once per 1024 polls.
                 const unsigned long long want = fa.tag + (unsigned long long)c;
                 unsigned spins = 0;
+                unsigned long long t0 = 0;
                 while (__hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want) {
                     __builtin_amdgcn_s_sleep(1);
-                    ++spins;
-                    if ((spins & 1023u) == 0 &&
-                        (spins > (1u << 20) ||
-                         __hip_atomic_load(fa.cnt + BH * 4, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == fa.tag)) {
-                        __hip_atomic_store(fa.cnt + BH * 4, fa.tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        ok = false;
-                        break;
+                    if ((++spins & 1023u) == 0) {
+                        const unsigned long long now = wall_clock64();
+                        if (t0 == 0) t0 = now;
+                        if (now - t0 > WAIT_LIMIT_TICKS ||
+                            __hip_atomic_load(fa.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == fa.tag) {
+                            __hip_atomic_store(fa.status, fa.tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            ok = false;
+                            break;
+                        }
                     }
                 }
                 // The last chunk is this counter's last reader: it takes the value away, so that a replay of
@@ -697,7 +681,6 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
                 for (int ct = 0; ct < 4; ++ct) h[ct] = float4_t{__builtin_nanf(""), __builtin_nanf(""), __builtin_nanf(""), __builtin_nanf("")};
             }
         }
-        FTS(2);
         bf16x8_t bhi[2], blo[2];
         split_sigma(h[0], h[1], bhi[0], blo[0]);
         split_sigma(h[2], h[3], bhi[1], blo[1]);
@@ -734,7 +717,6 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
 #pragma unroll
                 for (int e = 0; e < 4; ++e) dst[(16 * ct + 4 * g + e) * HEAD] = hn[ct][e];
         }
-        FTS(3);
         // O[i][v] = OI + Qt h: through an LDS tile so that every lane stores its own token row.  The tile is
         // written transposed, [value column][token], with one 8-byte store per accumulator tile, and read
         // back with the transposing load.
@@ -767,7 +749,6 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
                 *reinterpret_cast<bf16x8_t*>(fa.o + row + 32 * s + 8 * g) =
                     bf16x8_t{lo[0], lo[1], lo[2], lo[3], hi4[0], hi4[1], hi4[2], hi4[3]};
         }
-        FTS(4);
     }
 }
 
@@ -1121,8 +1102,11 @@ void chunk_items_kernel(SeqLayout L, int* __restrict__ items, const float* __res
                 }
             }
         }
-        if (c < nt) *reinterpret_cast<int4_t*>(items + 4 + 4 * pos) = int4_t{b, c, (int)mine.tok0, mine.len};
-        if (b == 0 && c == 0) items[0] = total;
+        // The list holds T / 64 + B entries, which covers every split of T tokens into B sequences; a table
+        // whose spans overlap can claim more chunks than that, and those are dropped.
+        const int capacity = (L.T >> 6) + L.B;
+        if (c < nt && pos < capacity) *reinterpret_cast<int4_t*>(items + 4 + 4 * pos) = int4_t{b, c, (int)mine.tok0, mine.len};
+        if (b == 0 && c == 0) items[0] = total < capacity ? total : capacity;
     }
     if (nt == 0 && dst != nullptr) {
         const int64_t per = (int64_t)L.H * STATE;
@@ -1145,7 +1129,7 @@ hipError_t launch_chunk_items(const SeqLayout& L, void* items, const float* src,
 TailFill tail_of_output(const SeqArgs& p) {
     TailFill t{};
     t.p[0] = p.o; t.n = 1;
-    t.row_bytes = (int64_t)p.H * p.N * (p.dtype == RWKV7_DTYPE_BF16 ? 2 : 4);
+    t.row_bytes = (int64_t)p.H * p.N * (p.dtype == RWKV7_DTYPE_F32 ? 4 : 2);     // bf16 and float16: 2 bytes
     return t;
 }
 
@@ -1160,12 +1144,16 @@ SeqLayout seq_layout(const SeqArgs& p, const void* ws) {
 
 size_t fwd_chunk_workspace_bytes(int B, int T, int H, bool varlen) {
     const int64_t nchunks = chunk_records(B, T, H, varlen);
-    // qt, pp, oi, qc: 4096 bf16 each; eg: 64 float
-    return (size_t)(nchunks * (4 * 4096 * 2 + 64 * 4)) + (varlen ? chunk_items_bytes(B, T) : 0);
+    // qt, pp, oi, qc: 4096 bf16 each; eg: 64 float; then the launch's 16-byte status record (padded to 256)
+    return (size_t)(nchunks * (4 * 4096 * 2 + 64 * 4)) + 256 + (varlen ? chunk_items_bytes(B, T) : 0);
+}
+
+size_t fwd_chunk_status_offset(int B, int T, int H, bool varlen) {
+    return (size_t)(chunk_records(B, T, H, varlen) * (4 * 4096 * 2 + 64 * 4)) + (varlen ? chunk_items_bytes(B, T) : 0);
 }
 
 namespace {
-struct ChunkWs { bf16_t *qt, *pp, *oi, *qc; float* eg; int64_t nchunks; SeqLayout L; };
+struct ChunkWs { bf16_t *qt, *pp, *oi, *qc; float* eg; unsigned long long* status; int64_t nchunks; SeqLayout L; };
 ChunkWs carve(const SeqArgs& p, void* ws) {
     ChunkWs c;
     c.nchunks = chunk_records(p.B, p.T, p.H, p.cu != nullptr);
@@ -1176,6 +1164,7 @@ ChunkWs carve(const SeqArgs& p, void* ws) {
     c.oi = reinterpret_cast<bf16_t*>(base + c.nchunks * 16384);
     c.qc = reinterpret_cast<bf16_t*>(base + c.nchunks * 24576);
     c.eg = reinterpret_cast<float*>(base + c.nchunks * 32768);
+    c.status = reinterpret_cast<unsigned long long*>(base + c.nchunks * (32768 + 256));
     return c;
 }
 }  // namespace
@@ -1195,10 +1184,34 @@ hipError_t launch_summary_kernel(const SeqArgs& p, int64_t nchunks, bf16_t* qt, 
 }
 }  // namespace
 
+namespace {
+// 64-bit mix (splitmix64 finaliser)
+inline unsigned long long mix64(unsigned long long z) {
+    z += 0x9e3779b97f4a7c15ull;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    return z ^ (z >> 31);
+}
+// A fresh pseudo-random tag per launch: process-wide sequence number, mixed with a per-process seed.
+unsigned long long next_launch_tag() {
+    static std::atomic<unsigned long long> seq{0};
+    static const unsigned long long seed =
+        mix64((unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count() ^
+              (unsigned long long)reinterpret_cast<uintptr_t>(&seq));
+    // never 0 or 1: a status record of zeros means "no launch has written here", and tag - 1 must differ from it
+    for (;;) {
+        const unsigned long long t = mix64(seed + seq.fetch_add(1, std::memory_order_relaxed));
+        if (t > 1ull) return t;
+    }
+}
+}  // namespace
+
 hipError_t launch_fwd_chunk_summary(const SeqArgs& p, void* ws, hipStream_t stream) {
     const ChunkWs c = carve(p, ws);
     FusedArgs fa{};
     fa.u = static_cast<const bf16_t*>(p.u6);
+    fa.status = c.status;              // this form cannot give up: the record only says that a launch wrote it
+    fa.tag = next_launch_tag();
     return p.u6 ? launch_summary_kernel<MODE_FWD, true>(p, c.nchunks, c.qt, c.pp, c.oi, c.qc, c.eg, c.L, fa, stream)
                 : launch_summary_kernel<MODE_FWD, false>(p, c.nchunks, c.qt, c.pp, c.oi, c.qc, c.eg, c.L, fa, stream);
 }
@@ -1241,28 +1254,14 @@ hipError_t launch_fwd_chunk(const SeqArgs& p, void* ws, hipStream_t stream) {
     return launch_fwd_chunk_scan(p, ws, stream);
 }
 
-namespace {
-// 64-bit mix (splitmix64 finaliser)
-inline unsigned long long mix64(unsigned long long z) {
-    z += 0x9e3779b97f4a7c15ull;
-    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
-    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
-    return z ^ (z >> 31);
+size_t fwd_fused_status_offset(int B, int T, int H, bool varlen) {
+    return (size_t)B * H * 32 + (varlen ? chunk_items_bytes(B, T) : 0);
 }
-// A fresh pseudo-random tag per launch: process-wide sequence number, mixed with a per-process seed.
-unsigned long long next_launch_tag() {
-    static std::atomic<unsigned long long> seq{0};
-    static const unsigned long long seed =
-        mix64((unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count() ^
-              (unsigned long long)reinterpret_cast<uintptr_t>(&seq));
-    return mix64(seed + seq.fetch_add(1, std::memory_order_relaxed));
-}
-}  // namespace
 
 size_t fwd_fused_workspace_bytes(int B, int T, int H, bool varlen) {
     const size_t bh = (size_t)B * H;
-    // 8-byte counters (one per head and value tile, plus the give-up flag), then two state slots per head
-    return ((bh * 32 + 8 + 255) / 256) * 256 + 2 * bh * 4096 * 4 + (varlen ? chunk_items_bytes(B, T) : 0);
+    // 8-byte counters (one per head and value tile), a 16-byte status record, then two state slots per head
+    return ((bh * 32 + 16 + 255) / 256) * 256 + 2 * bh * 4096 * 4 + (varlen ? chunk_items_bytes(B, T) : 0);
 }
 
 hipError_t launch_fwd_fused(const SeqArgs& p, void* ws, hipStream_t stream) {
@@ -1278,7 +1277,8 @@ hipError_t launch_fwd_fused(const SeqArgs& p, void* ws, hipStream_t stream) {
     fa.h0 = p.h0; fa.h0_batch_stride = p.h0_batch_stride; fa.h0_map = p.h0_map; fa.n_state = p.n_state;
     fa.o = (bf16_t*)p.o; fa.ht = p.ht;
     fa.cnt = reinterpret_cast<unsigned long long*>(base);
-    fa.hbuf = reinterpret_cast<float*>(base + (((size_t)BH * 32 + 8 + 255) / 256) * 256);
+    fa.hbuf = reinterpret_cast<float*>(base + (((size_t)BH * 32 + 16 + 255) / 256) * 256);
+    fa.status = fa.cnt + (size_t)BH * 4;
     // The hand-off counters are compared for EQUALITY with tag + chunk index, so whatever the workspace
     // holds on entry (an earlier launch's counters, or anything else) reads as "not there yet" unless it
     // equals one specific 64-bit value, and no clearing launch is needed in front of the kernel.  A

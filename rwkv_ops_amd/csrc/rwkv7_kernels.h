@@ -37,6 +37,11 @@ hipError_t launch_fwd_chunk(const SeqArgs& p, void* ws, hipStream_t stream);
 // the same forward as ONE kernel: each chunk's workgroup applies its summary to the state it receives
 // from the previous chunk's workgroup and hands the new state on (ws: fwd_fused_workspace_bytes)
 size_t fwd_fused_workspace_bytes(int B, int T, int H, bool varlen = false);
+// Byte offset, within the workspace of either form, of the launch's 16-byte status record (two 64-bit
+// words): [1] = the launch's tag (never 0), [0] = that tag if a hand-off wait of the one-kernel form timed
+// out and the outputs were poisoned, anything else otherwise.
+size_t fwd_fused_status_offset(int B, int T, int H, bool varlen = false);
+size_t fwd_chunk_status_offset(int B, int T, int H, bool varlen = false);
 hipError_t launch_fwd_fused(const SeqArgs& p, void* ws, hipStream_t stream);
 // its two halves: the parallel per-chunk summaries (reads r..b, fills ws) and the serial scan
 // (reads ws and h0, writes o and ht)

@@ -12,6 +12,8 @@ _CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(_CSRC, "librwkv7_mi355x.so")
 
 DTYPE_BF16, DTYPE_F32, DTYPE_F16 = 0, 1, 2
+NO_STATUS_RECORD = ctypes.c_size_t(-1).value
+FWD_DONE, FWD_GAVE_UP, FWD_NO_LAUNCH = 0, 1, 2
 ABI_VERSION = 1
 
 _P, _I, _I64, _SZ = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_size_t
@@ -21,6 +23,9 @@ SIGNATURES = {
     "rwkv7_abi_version": (_I, []),
     "rwkv7_status_string": (ctypes.c_char_p, [_I]),
     "rwkv7_fwd_workspace_bytes": (_SZ, [_I, _I, _I, _I]),
+    "rwkv7_fwd_status_offset": (_SZ, [_I, _I, _I, _I]),
+    "rwkv7_fwd_varlen_status_offset": (_SZ, [_I, _I, _I, _I]),
+    "rwkv7_fwd_status": (_I, [_P]),
     "rwkv7_fwd": (_I, [_P] * 6 + [_P, _I64, _P, _P] + [_I] * 6 + [_P, _SZ, _P]),
     "rwkv7_fwd_gather": (_I, [_P] * 6 + [_P, _I, _P, _P, _P] + [_I] * 6 + [_P, _SZ, _P]),
     "rwkv7_decode_step_gather": (_I, [_P] * 6 + [_P, _I, _P, _P, _P] + [_I] * 5 + [_P]),

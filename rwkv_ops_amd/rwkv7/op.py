@@ -390,6 +390,15 @@ def _compute_dtype(r: torch.Tensor, T: int = 0) -> torch.dtype:
     return torch.bfloat16
 
 
+def _out_dtype(r: torch.Tensor) -> torch.dtype:
+    """The dtype of ``out``, whatever the sequence length: float32 for float32 / float64 inputs, float16 for
+    float16 inputs (computed from bfloat16 operands beyond HALF_NATIVE_MAX_T tokens and rounded back),
+    bfloat16 for everything else."""
+    if r.dtype in (torch.float32, torch.float64):
+        return torch.float32
+    return torch.float16 if r.dtype == torch.float16 else torch.bfloat16
+
+
 def _prepare(x: torch.Tensor, dtype: torch.dtype, head_first: bool) -> torch.Tensor:
     if head_first:                                   # [B, H, T, K] -> [B, T, H, K]
         x = x.permute(0, 2, 1, 3)
@@ -476,6 +485,11 @@ def generalized_delta_rule(
 ):
     """RWKV7 generalized delta rule on MI355X; signature of torch_op.py:458-468 plus ``state_map``.
 
+    ``out`` has the dtype of the inputs for bfloat16, float16 and float32 inputs, whatever T is (the
+    reference's kernel path returns bfloat16 for all of them, torch_op.py:451-455,486); float16 sequences of
+    more than 12 tokens are computed from bfloat16-rounded operands, as the reference does, and ``out`` is
+    rounded back to float16.
+
     ``w`` is the raw decay argument: the per-step decay is ``exp(-exp(w))``
     (torch_op.py:433-434), so padded positions use ``w += (1 - mask) * -1e9`` together
     with zeroed r, k, v, a, b (/root/reference/README.md:89-98).
@@ -509,6 +523,8 @@ def generalized_delta_rule(
         out, state = _fwd_impl(r_, w_, k_, v_, a_, b_, h0, bool(output_final_state), smap)
     else:
         out, state = torch.ops.rwkv_ops_amd.rwkv7_fwd(r_, w_, k_, v_, a_, b_, h0, bool(output_final_state), smap)
+    if out.dtype != _out_dtype(r):
+        out = out.to(_out_dtype(r))
     if head_first:
         out = out.permute(0, 2, 1, 3)
     if output_final_state:
@@ -542,6 +558,8 @@ def _generalized_delta_rule_varlen(r, w, k, v, a, b, initial_state, output_final
     else:
         out, state = torch.ops.rwkv_ops_amd.rwkv7_fwd_varlen(r_, w_, k_, v_, a_, b_, h0,
                                                              bool(output_final_state), cu)
+    if out.dtype != _out_dtype(r):
+        out = out.to(_out_dtype(r))
     if output_final_state:
         return out, state
     return out

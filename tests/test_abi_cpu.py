@@ -148,3 +148,40 @@ def test_float16_is_a_dtype_only_where_a_kernel_reads_it():
     # accepted as a dtype by the decode step: the next check (head size, null pointer) is what answers
     assert lib.rwkv7_decode_step(x, x, x, x, x, x, None, 0, x, None, 2, 2, 32, 32, 2, None) == -3
     assert lib.rwkv7_decode_step(None, x, x, x, x, x, None, 0, x, None, 2, 2, 64, 64, 2, None) == -1
+
+
+def test_forward_status_record_on_a_host_image():
+    """rwkv7_fwd_status reads a HOST copy of the 16-byte record [flag, tag] that a chunked forward leaves in
+    its workspace; the offsets of the record lie inside the workspace of the form the call would choose."""
+    lib = _lib.load()
+    rec = (ctypes.c_uint64 * 2)
+
+    def status(flag, tag):
+        return lib.rwkv7_fwd_status(ctypes.cast(rec(flag, tag), ctypes.c_void_p))
+    assert status(0, 0) == _lib.FWD_NO_LAUNCH                        # a fresh (zeroed) workspace
+    tag = 0x9e3779b97f4a7c15
+    assert status(tag - 1, tag) == _lib.FWD_DONE                     # what the first workgroup writes
+    assert status(tag, tag) == _lib.FWD_GAVE_UP                      # what a wave that stopped waiting writes
+    assert status(12345, tag) == _lib.FWD_DONE                       # anything but the tag itself
+    assert lib.rwkv7_fwd_status(None) == -1
+    # a workspace image built on the host: zeros, then the record of a finished launch at the documented offset
+    for B, T, H in ((8, 4096, 32), (1, 300, 4)):                     # one-kernel form, two-kernel form
+        size = lib.rwkv7_fwd_workspace_bytes(B, T, H, 0)
+        off = lib.rwkv7_fwd_status_offset(B, T, H, 0)
+        assert off % 16 == 0 and off + 16 <= size
+        image = bytearray(size)
+        view = (ctypes.c_char * size).from_buffer(image)
+        assert lib.rwkv7_fwd_status(ctypes.cast(ctypes.addressof(view) + off, ctypes.c_void_p)) == _lib.FWD_NO_LAUNCH
+        image[off:off + 16] = (tag - 1).to_bytes(8, "little") + tag.to_bytes(8, "little")
+        assert lib.rwkv7_fwd_status(ctypes.cast(ctypes.addressof(view) + off, ctypes.c_void_p)) == _lib.FWD_DONE
+        image[off:off + 8] = tag.to_bytes(8, "little")
+        assert lib.rwkv7_fwd_status(ctypes.cast(ctypes.addressof(view) + off, ctypes.c_void_p)) == _lib.FWD_GAVE_UP
+        del view
+    n_seq, T, H = 5, 1000, 32
+    off = lib.rwkv7_fwd_varlen_status_offset(n_seq, T, H, 0)
+    assert off % 16 == 0 and off + 16 <= lib.rwkv7_fwd_varlen_workspace_bytes(n_seq, T, H, 0)
+    # calls that run no chunked kernel leave no record
+    assert lib.rwkv7_fwd_status_offset(8, 12, 32, 0) == _lib.NO_STATUS_RECORD
+    assert lib.rwkv7_fwd_status_offset(8, 4096, 32, 1) == _lib.NO_STATUS_RECORD
+    assert lib.rwkv7_fwd_varlen_status_offset(5, 1000, 32, 2) == _lib.NO_STATUS_RECORD
+

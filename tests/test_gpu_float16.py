@@ -41,7 +41,47 @@ def test_float16_long_sequences_take_the_bf16_kernels(device):
     xs = make_inputs(2, 200, 3, 64, seed=712, dtype=torch.float16)
     o_ref, s_ref = native_c.run(*[x.to(torch.bfloat16) for x in xs[:6]], xs[6])
     o, s = rwkv_ops_amd.generalized_delta_rule(*[x.to(device) for x in xs])
+    assert o.dtype == torch.float16
     assert rel_l2(o, o_ref) < 5e-3 and rel_l2(s, s_ref) < 5e-3
+
+
+def test_float16_output_dtype_does_not_depend_on_the_length(device):
+    """T = 12 runs the float16 kernels, T = 13 the bf16 chunked ones; `out` is float16 either way, and so is
+    the output of a packed call and of a decode step."""
+    for T in (1, 12, 13, 100):
+        xs = make_inputs(2, T, 3, 64, seed=720 + T, dtype=torch.float16)
+        o, s = rwkv_ops_amd.generalized_delta_rule(*[x.to(device) for x in xs])
+        assert o.dtype == torch.float16 and s.dtype == torch.float32, T
+        ref_in = xs[:6] if T <= 12 else [x.to(torch.bfloat16) for x in xs[:6]]
+        o_ref, s_ref = native_c.run(*ref_in, xs[6])
+        assert rel_l2(o, o_ref) < 5e-3 and rel_l2(s, s_ref) < 5e-3, T
+    xs = make_inputs(1, 90, 3, 64, seed=719, dtype=torch.float16, h0=False)
+    o = rwkv_ops_amd.generalized_delta_rule(*[x.to(device) for x in xs[:6]], cu_seqlens=[0, 40, 90],
+                                            output_final_state=False)
+    assert o.dtype == torch.float16
+
+
+def test_float16_packed_rows_behind_the_last_sequence(device):
+    """rwkv7_fwd_varlen with RWKV7_DTYPE_F16 through the C ABI and a table that ends before T_total: the rows
+    of o behind the last sequence are zero-filled -- 2 bytes per element, so the fill ends where o ends (o is
+    carved out of a larger buffer of sentinels, which must survive) -- for K = 64 and 128."""
+    lib = _lib.load()
+    for N in (64, 128):
+        T, H, used = 50, 3, 33
+        xs = [x.to(device) for x in make_inputs(1, T, H, N, seed=730 + N, dtype=torch.float16, h0=False)[:6]]
+        cu = torch.tensor([0, 20, used], dtype=torch.int32, device=device)
+        n = T * H * N
+        buf = torch.full((3 * n,), 7.0, dtype=torch.float16, device=device)
+        o = buf[n:2 * n]
+        rc = lib.rwkv7_fwd_varlen(*[x.data_ptr() for x in xs], cu.data_ptr(), 2, None, 0, o.data_ptr(), None,
+                                  T, H, N, N, _lib.DTYPE_F16, None, 0, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        torch.cuda.synchronize()
+        assert bool((buf[:n] == 7.0).all()) and bool((buf[2 * n:] == 7.0).all()), "wrote outside o"
+        o = o.view(1, T, H, N)
+        assert bool((o[:, used:] == 0).all()), "rows behind the last sequence must be zero"
+        o_ref, _ = native_c.run(*[x[:, 20:used].cpu() for x in xs], None)
+        assert rel_l2(o[:, 20:used], o_ref) < 2e-3
 
 
 def test_float16_is_refused_where_no_kernel_reads_it(device):
