@@ -64,6 +64,7 @@ extern "C" {
 #define RWKV7_ERR_WORKSPACE     -6   /* workspace NULL, misaligned (256 B) or smaller than *_workspace_bytes */
 #define RWKV7_ERR_ALIGNMENT     -7   /* a tensor pointer is not 16-byte aligned */
 #define RWKV7_ERR_UNSUPPORTED   -8   /* combination not built (see the function's comment) */
+#define RWKV7_ERR_TOO_LARGE     -9   /* rwkv7_fwd_noalloc: B*H > RWKV7_NOALLOC_MAX_BH */
 
 int rwkv7_abi_version(void);
 
@@ -94,6 +95,31 @@ int rwkv7_fwd(const void* r, const void* w, const void* k, const void* v,
               void* o, float* ht,
               int B, int T, int H, int K, int V, int dtype,
               void* ws, size_t ws_bytes, void* stream);
+
+/* ---- the forward without a workspace argument ---------------------------------------
+ * No counterpart in the reference.  For callers that cannot allocate device memory
+ * around the call -- code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc -- and so cannot provide rwkv7_fwd's workspace: the same forward,
+ * same arguments and results, with the workspace taken from a static device array
+ * inside the library (8.01 MiB, held on every GPU the library is loaded on until the
+ * process ends).  That array holds the one-kernel form's hand-off slots and counters
+ * for up to RWKV7_NOALLOC_MAX_BH (batch, head) sequences, so B*H beyond that is refused
+ * with RWKV7_ERR_TOO_LARGE; T is not limited.  bf16 with T > 12 always takes the
+ * one-kernel chunked form here (rwkv7_fwd prefers two kernels below 96 sequences, whose
+ * workspace grows with T); T == 1, T <= 12, float32, float16 and K = V = 128 take the
+ * same kernels as in rwkv7_fwd, which need no workspace.  The call itself allocates
+ * nothing and calls no allocating routine; its first call on a device looks the
+ * array's address up (hipGetSymbolAddress), so make that one outside a capture.  All
+ * calls on one GPU share the array: two of them that overlap in time (different
+ * streams, or graphs replayed concurrently) race and give wrong results; calls on one
+ * stream are ordered and safe.  Nothing in the array needs clearing between calls:
+ * every launch tags its counters with a fresh 64-bit value (see rwkv7_fwd_status). */
+#define RWKV7_NOALLOC_MAX_BH 256
+int rwkv7_fwd_noalloc(const void* r, const void* w, const void* k, const void* v,
+                      const void* a, const void* b,
+                      const float* h0, int64_t h0_batch_stride,
+                      void* o, float* ht,
+                      int B, int T, int H, int K, int V, int dtype, void* stream);
 
 /* ---- did a chunked forward finish? ------------------------------------------------
  * The one-kernel chunked forward hands each (batch, head) state from one 64-token

@@ -4,6 +4,8 @@
 #include "../../include/rwkv6_mi355x.h"
 #include "rwkv7_kernels.h"
 
+#include <atomic>
+
 using rwkv7::SeqArgs;
 
 namespace {
@@ -63,6 +65,7 @@ const char* rwkv7_status_string(int status) {
         case RWKV7_ERR_WORKSPACE: return "workspace is NULL, not 256-byte aligned or too small";
         case RWKV7_ERR_ALIGNMENT: return "tensor pointers must be 16-byte aligned";
         case RWKV7_ERR_UNSUPPORTED: return "this combination of arguments is not built";
+        case RWKV7_ERR_TOO_LARGE: return "rwkv7_fwd_noalloc: B*H exceeds RWKV7_NOALLOC_MAX_BH (256), the size of the library's static scratch";
         default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
@@ -142,6 +145,55 @@ int rwkv7_fwd(const void* r, const void* w, const void* k, const void* v, const 
     if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return RWKV7_ERR_WORKSPACE;
     if (use_fused_forward(B, H)) return (int)rwkv7::launch_fwd_fused(p, ws, static_cast<hipStream_t>(stream));
     return (int)rwkv7::launch_fwd_chunk(p, ws, static_cast<hipStream_t>(stream));
+}
+
+/* ---- the forward for callers that may not allocate -------------------------------------------- */
+namespace {
+// The one-kernel forward's workspace (hand-off counters, status record, two state slots per (batch, head))
+// for RWKV7_NOALLOC_MAX_BH sequences, held by every GPU the library is loaded on until the process ends.
+constexpr size_t SCRATCH_BYTES =
+    (((size_t)RWKV7_NOALLOC_MAX_BH * 32 + 16 + 255) / 256) * 256 + 2 * (size_t)RWKV7_NOALLOC_MAX_BH * 4096 * 4;
+static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
+// The array's name is a host-side stand-in; its device address differs per GPU and is looked up once per
+// device (with that device current) and kept here.
+constexpr int MAX_DEVICES = 64;
+std::atomic<void*> scratch_ptr[MAX_DEVICES];
+
+int scratch_on_current_device(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= MAX_DEVICES) return RWKV7_ERR_UNSUPPORTED;
+    void* p = scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (p == nullptr || (reinterpret_cast<uintptr_t>(p) & 255u) != 0) return RWKV7_ERR_WORKSPACE;
+        scratch_ptr[dev].store(p, std::memory_order_release);    // (two threads racing here store the same address)
+    }
+    *out = p;
+    return RWKV7_OK;
+}
+}  // namespace
+
+int rwkv7_fwd_noalloc(const void* r, const void* w, const void* k, const void* v, const void* a,
+                      const void* b, const float* h0, int64_t h0_batch_stride, void* o, float* ht,
+                      int B, int T, int H, int K, int V, int dtype, void* stream)
+{
+    int rc = check_seq(r, w, k, v, a, b, h0, h0_batch_stride, o, ht, B, T, H, K, V, dtype, true, true);
+    if (rc != RWKV7_OK) return rc;
+    SeqArgs p = pack(r, w, k, v, a, b, h0, h0_batch_stride, o, ht, B, T, H, dtype, K);
+    // the same routing as rwkv7_fwd for the kernels that use no workspace
+    if (T == 1) return (int)rwkv7::launch_decode(p, static_cast<hipStream_t>(stream));
+    if (dtype != RWKV7_DTYPE_BF16 || K == 128 || T <= RECURRENT_MAX_T)
+        return (int)rwkv7::launch_fwd_recurrent(p, static_cast<hipStream_t>(stream));
+    // Always the one-kernel form: its workspace does not grow with T.
+    if ((int64_t)B * H > RWKV7_NOALLOC_MAX_BH || rwkv7::fwd_fused_workspace_bytes(B, T, H) > SCRATCH_BYTES)
+        return RWKV7_ERR_TOO_LARGE;
+    void* ws = nullptr;
+    rc = scratch_on_current_device(&ws);
+    if (rc != RWKV7_OK) return rc;
+    return (int)rwkv7::launch_fwd_fused(p, ws, static_cast<hipStream_t>(stream));
 }
 
 /* ---- the same two calls with the initial states gathered through a map --------------------------- */

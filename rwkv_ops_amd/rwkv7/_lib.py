@@ -27,6 +27,7 @@ SIGNATURES = {
     "rwkv7_fwd_varlen_status_offset": (_SZ, [_I, _I, _I, _I]),
     "rwkv7_fwd_status": (_I, [_P]),
     "rwkv7_fwd": (_I, [_P] * 6 + [_P, _I64, _P, _P] + [_I] * 6 + [_P, _SZ, _P]),
+    "rwkv7_fwd_noalloc": (_I, [_P] * 6 + [_P, _I64, _P, _P] + [_I] * 6 + [_P]),
     "rwkv7_fwd_gather": (_I, [_P] * 6 + [_P, _I, _P, _P, _P] + [_I] * 6 + [_P, _SZ, _P]),
     "rwkv7_decode_step_gather": (_I, [_P] * 6 + [_P, _I, _P, _P, _P] + [_I] * 5 + [_P]),
     "rwkv7_fwd_chunk_workspace_bytes": (_SZ, [_I, _I, _I, _I]),

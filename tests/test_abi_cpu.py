@@ -32,7 +32,7 @@ def test_every_declared_symbol_is_exported():
 
 
 def test_status_strings():
-    for code in range(-8, 1):
+    for code in range(-9, 1):
         s = _lib.status_string(code)
         assert s and "unknown" not in s
     assert "unknown" in _lib.status_string(-99)
@@ -185,3 +185,17 @@ def test_forward_status_record_on_a_host_image():
     assert lib.rwkv7_fwd_status_offset(8, 4096, 32, 1) == _lib.NO_STATUS_RECORD
     assert lib.rwkv7_fwd_varlen_status_offset(5, 1000, 32, 2) == _lib.NO_STATUS_RECORD
 
+
+def test_noalloc_forward_argument_errors_do_not_launch():
+    lib = _lib.load()
+    x = 0x1000
+
+    def fwd(B=8, T=100, H=32, K=64, dtype=0, r=x, o=x):
+        return lib.rwkv7_fwd_noalloc(r, x, x, x, x, x, None, 0, o, None, B, T, H, K, K, dtype, None)
+    assert fwd(B=9) == -9                                            # 288 sequences: beyond the static scratch
+    assert fwd(B=1, H=257) == -9
+    assert "256" in _lib.status_string(-9)
+    assert fwd(r=None) == -1 and fwd(o=None) == -1
+    assert fwd(K=32) == -3
+    assert fwd(dtype=9) == -2
+    assert fwd(T=0) == -4
