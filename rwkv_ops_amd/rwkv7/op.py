@@ -407,17 +407,26 @@ def _prepare(x: torch.Tensor, dtype: torch.dtype, head_first: bool) -> torch.Ten
     return x.to(dtype).contiguous()
 
 
-def _as_state_map(state_map, B: int, n_state: int, device: torch.device) -> torch.Tensor:
-    """int32 ``[B]`` on ``device`` with entries in ``[0, n_state)`` (checked, as the reference's RWKV6
-    operator checks its state_map, torch_rwkv_kernel.py:293-297; the check reads the map back)."""
+def _as_state_map(state_map, B: int, n_state: int, device: torch.device, distinct: bool = False) -> torch.Tensor:
+    """int32 ``[B]`` on ``device``.  A list or a CPU tensor is checked (entries in ``[0, n_state)``, as the
+    reference's RWKV6 operator checks its state_map, torch_rwkv_kernel.py:293-297; ``distinct``: no entry
+    twice).  A tensor already on the device is taken as it is: reading it back would stall the stream on every
+    decode step and cannot happen under graph capture; the kernels clamp what they read, so a bad entry cannot
+    fault, and distinct entries are then the caller's contract."""
     if isinstance(state_map, (list, tuple)):
         state_map = torch.tensor(state_map, dtype=torch.int32)
     if not isinstance(state_map, torch.Tensor) or state_map.dtype not in (torch.int32, torch.int64):
         raise ValueError("state_map must be a list or an int32/int64 tensor of shape [B]")
     if tuple(state_map.shape) != (B,):
         raise ValueError(f"state_map must have shape [{B}], got {tuple(state_map.shape)}")
-    if bool((state_map < 0).any()) or bool((state_map >= n_state).any()):
-        raise ValueError(f"state_map entries must lie in [0, {n_state})")
+    if not state_map.is_cuda:
+        m = state_map.tolist()
+        if any(e < 0 or e >= n_state for e in m):
+            raise ValueError(f"state_map entries must lie in [0, {n_state})")
+        if distinct and len(set(m)) != B:
+            raise ValueError("state_map entries must be distinct for an in-place update")
+    if state_map.device == device and state_map.dtype == torch.int32 and state_map.is_contiguous():
+        return state_map
     return state_map.to(device=device, dtype=torch.int32).contiguous()
 
 
@@ -572,7 +581,9 @@ def rwkv7_decode_step(r, w, k, v, a, b, state, state_map=None):
     Equivalent to ``generalized_delta_rule`` with T = 1 and ``initial_state=state``, without
     allocating a second state.  With ``state_map`` (list or int tensor ``[B]``, distinct entries)
     ``state`` is a pool ``[n_state, H, 64, 64]`` and row b reads and updates ``state[state_map[b]]``:
-    the serving loop's slot table, no gather or scatter of states around the step."""
+    the serving loop's slot table, no gather or scatter of states around the step.  A map given as a list
+    or a CPU tensor is checked; an int32 tensor on the device is used as it is, without any read-back, so
+    the step never synchronises and can be captured into a graph."""
     squeeze = r.dim() == 4
     xs = [x[:, 0] if squeeze else x for x in (r, w, k, v, a, b)]
     for x in xs:
@@ -584,9 +595,7 @@ def rwkv7_decode_step(r, w, k, v, a, b, state, state_map=None):
     if state_map is not None:
         if N not in HEAD_SIZES or state.dim() != 4 or tuple(state.shape[1:]) != (H, N, N):
             raise ValueError(f"state must be [n_state, {H}, {N}, {N}] with a head size in {HEAD_SIZES}, got {tuple(state.shape)}")
-        smap = _as_state_map(state_map, B, state.shape[0], state.device)
-        if int(torch.unique(smap).numel()) != B:
-            raise ValueError("state_map entries must be distinct for an in-place update")
+        smap = _as_state_map(state_map, B, state.shape[0], state.device, distinct=True)
     elif N not in HEAD_SIZES or tuple(state.shape) != (B, H, N, N):
         raise ValueError(f"state must be [{B}, {H}, {N}, {N}] with a head size in {HEAD_SIZES}, got {tuple(state.shape)}")
     dt = _compute_dtype(xs[0], 1)

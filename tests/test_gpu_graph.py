@@ -65,6 +65,63 @@ def test_decode_under_graph_replay(device):
         assert torch.equal(o_g, o_e) and torch.equal(state_g, state_e)
 
 
+def test_decode_pool_under_graph_replay(device):
+    """A decode step over a pool of states with the slot table on the device: nothing in the call reads the
+    table back (a read-back cannot be captured), the replays follow the table's current contents, and every
+    replay equals the eager call and the CPU oracle on the gathered states."""
+    from oracle import native_c
+    from rwkv_ops_amd.synthetic import rel_l2
+    B, H, steps, n_state = 5, 4, 3, 9
+    xs = make_inputs(B, steps, H, 64, seed=51, dtype=torch.bfloat16)
+    seq = [x.to(device) for x in xs[:6]]
+    g = torch.Generator().manual_seed(52)
+    pool_cpu = 0.1 * torch.randn(n_state, H, 64, 64, generator=g)
+    pool_g, pool_e = pool_cpu.to(device), pool_cpu.to(device)
+    maps = [[8, 0, 3, 5, 1], [2, 7, 3, 0, 6], [4, 5, 6, 7, 8]]
+    smap = torch.tensor(maps[0], dtype=torch.int32, device=device)
+    stat = [s[:, 0].contiguous().clone() for s in seq]
+    rwkv_ops_amd.rwkv7_decode_step(*stat, pool_g.clone(), state_map=smap)            # warm-up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        o_g = rwkv_ops_amd.rwkv7_decode_step(*stat, pool_g, state_map=smap)
+    pool_g.copy_(pool_cpu)
+    for t in range(steps):
+        for dst, s in zip(stat, seq):
+            dst.copy_(s[:, t])
+        smap.copy_(torch.tensor(maps[t], dtype=torch.int32))
+        before = pool_e.cpu()
+        graph.replay()
+        torch.cuda.synchronize()
+        o_e = rwkv_ops_amd.rwkv7_decode_step(*[s[:, t].contiguous() for s in seq], pool_e, state_map=maps[t])
+        torch.cuda.synchronize()
+        assert torch.equal(o_g, o_e) and torch.equal(pool_g, pool_e)
+        o_ref, s_ref = native_c.run(*[x[:, t:t + 1] for x in xs[:6]], before[maps[t]])
+        assert rel_l2(o_g[:, None], o_ref) < 5e-3 and rel_l2(pool_g[maps[t]], s_ref) < 5e-3
+        untouched = [i for i in range(n_state) if i not in maps[t]]
+        assert torch.equal(pool_g[untouched].cpu(), before[untouched])
+
+
+def test_forward_with_a_device_state_map_under_graph_replay(device):
+    B, T, H, n_state = 4, 130, 32, 6
+    xs = make_inputs(B, T, H, 64, seed=53, dtype=torch.bfloat16)
+    dev = [x.to(device) for x in xs[:6]]
+    pool = (0.1 * torch.randn(n_state, H, 64, 64, generator=torch.Generator().manual_seed(54))).to(device)
+    smap = torch.tensor([5, 0, 0, 2], dtype=torch.int32, device=device)
+    rwkv_ops_amd.generalized_delta_rule(*dev, initial_state=pool, state_map=smap)    # warm-up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        o_g, s_g = rwkv_ops_amd.generalized_delta_rule(*dev, initial_state=pool, state_map=smap)
+    for m in ([1, 1, 4, 3], [0, 5, 2, 2]):
+        smap.copy_(torch.tensor(m, dtype=torch.int32))
+        graph.replay()
+        torch.cuda.synchronize()
+        o_e, s_e = rwkv_ops_amd.generalized_delta_rule(*dev, initial_state=pool, state_map=m)
+        torch.cuda.synchronize()
+        assert torch.equal(o_g, o_e) and torch.equal(s_g, s_e)
+
+
 def test_backward_under_graph_replay(device):
     B, T, H = 2, 200, 3
     sets = [make_inputs(B, T, H, 64, seed=60 + i, dtype=torch.bfloat16) for i in range(2)]
