@@ -44,6 +44,10 @@ N = 64
 # counter reads for a plain 1 GiB copy (FETCH_SIZE x2.000, WRITE_SIZE x1.000); the summary is
 # profiles/fwd_chunk_prefill_and_decode_traffic.txt.
 MEASURED_TRAFFIC_BYTES = 1480869460
+TRAFFIC_SOURCE = ("profiles/fwd_chunk_prefill_and_decode_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this "
+                  "command at B=8 T=4096 H=32; a constant, not measured in this run)")
+EXEC_FLOPS_SOURCE = ("profiles/fwd_chunk_prefill_mfma_counters.txt (SQ_INSTS_VALU_MFMA_MOPS_BF16: 118,784 flop per "
+                     "token-head; a constant, not measured in this run)")
 
 
 def algorithmic_bytes_prefill(B, T, H):
@@ -285,15 +289,23 @@ def main():
     del ws6, w6
 
     # ------------------------------------------------------------------ one long sequence (few heads: two-kernel form)
-    Bl, Tl, Hl = 1, 16384, 64
-    xl = [t.to(dev) for t in make_inputs(Bl, Tl, Hl, N, seed=3, dtype=torch.bfloat16)]
+    # BASELINE config 3: B=1, T=16384, H=64, zero initial state, the last 1024 tokens padded by the
+    # w += (1 - mask) * -1e9 convention with r, k, v, a, b zeroed (the inputs of tests/test_gpu_fullsize.py)
+    Bl, Tl, Hl, padl = 1, 16384, 64, 1024
+    xl = list(make_inputs(Bl, Tl, Hl, N, seed=1237, dtype=torch.bfloat16, h0=False))
+    maskl = torch.ones(Bl, Tl, 1, 1)
+    maskl[:, Tl - padl:] = 0
+    for i in (0, 2, 3, 4, 5):
+        xl[i] = (xl[i].float() * maskl).to(torch.bfloat16)
+    xl[1] = (xl[1].float() + (1 - maskl) * -1e9).to(torch.bfloat16)
+    xl = [t.to(dev) for t in xl[:6]]
     ol = torch.empty_like(xl[0])
     htl = torch.empty(Bl, Hl, N, N, dtype=torch.float32, device=dev)
     wsl_bytes = lib.rwkv7_fwd_workspace_bytes(Bl, Tl, Hl, 0)
     wsl = torch.empty(wsl_bytes, dtype=torch.uint8, device=dev)
 
     def long_fwd():
-        rc = lib.rwkv7_fwd(*[ptr(t) for t in xl[:6]], ptr(xl[6]), Hl * N * N, ptr(ol), ptr(htl),
+        rc = lib.rwkv7_fwd(*[ptr(t) for t in xl[:6]], None, 0, ptr(ol), ptr(htl),
                            Bl, Tl, Hl, N, N, 0, ptr(wsl), wsl_bytes, stream)
         assert rc == 0, rc
 
@@ -302,14 +314,30 @@ def main():
         assert rc == 0, rc
 
     def long_scan():
-        rc = lib.rwkv7_fwd_chunk_scan(ptr(xl[6]), Hl * N * N, ptr(ol), ptr(htl), Bl, Tl, Hl, N, N, 0,
+        rc = lib.rwkv7_fwd_chunk_scan(None, 0, ptr(ol), ptr(htl), Bl, Tl, Hl, N, N, 0,
                                       ptr(wsl), wsl_bytes, stream)
         assert rc == 0, rc
 
     ms_long, _ = time_gpu(long_fwd, args.steps, 3, torch)
     ms_long_summary, _ = time_gpu(long_summary, args.steps, 3, torch)
     ms_long_scan, _ = time_gpu(long_scan, args.steps, 3, torch)
+    long_bytes = 7 * Bl * Tl * Hl * N * 2 + Bl * Hl * N * N * 4      # no initial state to read
     del wsl, xl, ol
+
+    # ------------------------------------------------------------------ float32 inputs at the prefill shape
+    # float32 callers get float32 arithmetic (1e-4 against the reference's native path): the recurrent kernel,
+    # one token at a time with the state in registers
+    x32 = [t.float() for t in (r, w, k, v, a, b)]
+    o32 = torch.empty_like(x32[0])
+
+    def fwd_f32():
+        rc = lib.rwkv7_fwd(*[ptr(t) for t in x32], ptr(h0), H * N * N, ptr(o32), ptr(ht),
+                           B, T, H, N, N, 1, None, 0, stream)
+        assert rc == 0, rc
+
+    ms_f32, _ = time_gpu(fwd_f32, max(5, args.steps // 10), 2, torch)
+    f32_bytes = 7 * B * T * H * N * 4 + 2 * B * H * N * N * 4
+    del x32, o32
 
     # ------------------------------------------------------------------ CPU baseline (rank 0, N = 1)
     cpu = None
@@ -351,6 +379,23 @@ def main():
         except Exception as exc:                                  # the C build is optional for the bench
             cpu["c_port"] = {"error": str(exc)}
 
+        # BASELINE config 0 itself (B=1, T=256, H=4, float32, head_first=False, final state returned): the
+        # reference's own CPU-runnable case on all host cores, one warm-up call and the median of five
+        import statistics
+        torch.set_num_threads(os.cpu_count() or 1)
+        c0 = make_inputs(1, 256, 4, N, seed=1234, dtype=torch.float32)
+        orc.generalized_delta_rule(*c0[:6], c0[6])
+        times0 = []
+        for _ in range(5):
+            t0 = time.perf_counter()
+            orc.generalized_delta_rule(*c0[:6], c0[6])
+            times0.append(time.perf_counter() - t0)
+        med0 = statistics.median(times0)
+        cpu["config0"] = {"value": 256 / med0, "unit": "tokens/s", "cores": os.cpu_count() or 1,
+                          "sample": f"B=1,T=256,H=4 float32 (BASELINE config 0), torch restatement of the reference "
+                                    f"native loop, 1 warm-up + median of 5 calls, {med0 * 1e3:.1f} ms each"}
+        torch.set_num_threads(threads)
+
     out = {
         "metric": "rwkv7_prefill_tokens_per_s",
         "value": tokens_per_s,
@@ -370,12 +415,14 @@ def main():
                    "global_batch": B, "seq_len": T, "heads": H, "head_size": N},
         "roofline": {"bound": "hbm", "achieved": achieved / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK, "traffic": MEASURED_TRAFFIC_BYTES,
+                     "traffic_source": TRAFFIC_SOURCE,
                      "algorithmic_bytes": alg_bytes,
                      "kernel": "chunk_summary_kernel<MODE_FUSED> (one launch = one step)",
                      "kernel_ms": ms_fused,
                      "two_kernel_form": {"chunk_summary_kernel_ms": ms_summary, "chunk_scan_kernel_ms": ms_scan}},
         "mfma": {"algorithmic_tflops": alg_flops / (ms_step * 1e-3) / 1e12,
                  "algorithmic_frac_of_bf16_peak": alg_flops / (ms_step * 1e-3) / MFMA_BF16_PEAK,
+                 "executed_flops_source": EXEC_FLOPS_SOURCE,
                  "executed_tflops": exec_flops / (ms_step * 1e-3) / 1e12,
                  "executed_frac_of_bf16_peak": exec_flops / (ms_step * 1e-3) / MFMA_BF16_PEAK},
         "decode": {"workload": f"T=1 decode, B={Bd} H={Hd}, bf16 inputs, float32 state updated in place, "
@@ -398,11 +445,18 @@ def main():
                    "forward_ms": ms_packed_fwd, "forward_tokens_per_s": B * T / (ms_packed_fwd * 1e-3),
                    "forward_frac_of_hbm_peak": (alg_bytes + 2 * (n_seq - B) * H * N * N * 4) / (ms_packed_fwd * 1e-3) / HBM_PEAK,
                    "backward_ms": ms_packed_bwd, "backward_tokens_per_s": B * T / (ms_packed_bwd * 1e-3)},
-        "long_sequence": {"workload": f"one sequence, B={Bl} T={Tl} H={Hl} bf16 (rwkv7_fwd: per-chunk summaries, then the "
-                                      "value-split scan, the form for fewer than 96 heads)",
+        "long_sequence": {"workload": f"BASELINE config 3: one sequence, B={Bl} T={Tl} H={Hl} bf16, zero initial state, the "
+                                      f"last {padl} tokens masked by w += (1-mask)*-1e9 (rwkv7_fwd: per-chunk summaries, "
+                                      "then the value-split scan, the form for fewer than 96 heads)",
                           "ms": ms_long, "tokens_per_s": Bl * Tl / (ms_long * 1e-3),
+                          "algorithmic_bytes": long_bytes,
+                          "frac_of_hbm_peak": long_bytes / (ms_long * 1e-3) / HBM_PEAK,
                           "chunk_summary_kernel_ms": ms_long_summary, "chunk_scan_vsplit_kernel_ms": ms_long_scan,
                           "scan_us_per_chunk": ms_long_scan * 1e3 / (Tl // 64)},
+        "float32": {"workload": f"generalized_delta_rule on float32 inputs, B={B} T={T} H={H} (the float32 recurrent "
+                                "kernel: 1e-4 parity with the reference's native path)",
+                    "ms": ms_f32, "tokens_per_s": B * T / (ms_f32 * 1e-3), "us_per_token": ms_f32 * 1e3 / T,
+                    "algorithmic_bytes": f32_bytes, "frac_of_hbm_peak": f32_bytes / (ms_f32 * 1e-3) / HBM_PEAK},
         "rwkv6": {"workload": f"RWKV6 operator forward (rwkv6_fwd), B={B} T={T} H={H} bf16, float32 states in and out",
                   "ms": ms_rwkv6, "tokens_per_s": B * T / (ms_rwkv6 * 1e-3), "algorithmic_bytes": rwkv6_bytes,
                   "frac_of_hbm_peak": rwkv6_bytes / (ms_rwkv6 * 1e-3) / HBM_PEAK},

@@ -36,6 +36,12 @@ def make_inputs(B, T, H, N=64, *, seed=0, dtype=torch.float32, h0=True, h0_batch
     return r, w, k, v, a, b, state
 
 
+# Relative-L2 thresholds of the bf16 backward against float32 autograd through the oracle on the same rounded
+# inputs, per gradient (the reference states none; measured 2.9e-3 .. 5.1e-3, see tests/test_gpu_backward.py).
+GRAD_NAMES = ("dr", "dw", "dk", "dv", "da", "db", "dh0")
+GRAD_TOL = {"dr": 6e-3, "dw": 8e-3, "dk": 6e-3, "dv": 6e-3, "da": 1e-2, "db": 1e-2, "dh0": 6e-3}
+
+
 def rel_l2(x, ref):
     """Relative L2 error ``|x - ref| / |ref|`` in float64 (the parity metric)."""
     x = x.detach().double().cpu()
