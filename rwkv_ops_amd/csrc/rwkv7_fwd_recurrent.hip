@@ -39,8 +39,11 @@ void fwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
                           const T* __restrict__ v, const T* __restrict__ a, const T* __restrict__ b,
                           const float* __restrict__ h0, int64_t h0_batch_stride,
                           const int* __restrict__ h0_map, int n_state,
-                          T* __restrict__ o, float* __restrict__ ht, SeqLayout L)
+                          T* __restrict__ o, float* __restrict__ ht, SeqLayout L,
+                          float* __restrict__ seg_states = nullptr, int seg = 0)
 {
+    // seg_states (dense batches only): the state BEFORE token t is stored for every t that is a multiple of `seg`
+    // (a multiple of REC_TB), [workgroup][t / seg][N][N]: what the recurrent backward restarts from.  o may then be NULL.
     constexpr int VQ = CPW / 4;                  // lanes across a wave's columns, four columns each
     constexpr int ROWS = N / (64 / VQ);          // state rows per lane
     constexpr int NT = 64 * (N / CPW);           // threads
@@ -127,6 +130,12 @@ void fwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
         deposit();
         __syncthreads();
         request(t0 + REC_TB);
+        if (seg_states != nullptr && t0 % seg == 0) {
+            const int nseg = (T_len + seg - 1) / seg;
+            float* dst = seg_states + ((int64_t)blockIdx.x * nseg + t0 / seg) * (N * N) + tile;
+#pragma unroll
+            for (int i = 0; i < ROWS; ++i) *reinterpret_cast<float4_t*>(dst + i * N) = s[i];
+        }
         const int nt = T_len - t0 < REC_TB ? T_len - t0 : REC_TB;
 #pragma unroll 4
         for (int tt = 0; tt < nt; ++tt) {
@@ -163,7 +172,7 @@ void fwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
             }
             acc.x = reduce_row_groups<VQ>(acc.x); acc.y = reduce_row_groups<VQ>(acc.y);
             acc.z = reduce_row_groups<VQ>(acc.z); acc.w = reduce_row_groups<VQ>(acc.w);
-            if (ks == 0) {
+            if (ks == 0 && o != nullptr) {
                 const float ov[4] = {acc.x, acc.y, acc.z, acc.w};
                 Io<T>::store4(o + base + (t0 + tt) * step + CPW * part + 4 * vq, ov);
             }
@@ -182,6 +191,25 @@ static hipError_t launch_t(const SeqArgs& p, hipStream_t stream) {
         (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, (const T*)p.a, (const T*)p.b,
         p.h0, p.h0_batch_stride, p.h0_map, p.n_state, (T*)p.o, p.ht, seq_layout(p, nullptr));
     return hipGetLastError();
+}
+
+template <typename T, int N>
+static hipError_t launch_states_t(const SeqArgs& p, float* states, int seg, hipStream_t stream) {
+    fwd_recurrent_kernel<T, N><<<dim3((unsigned)(p.B * p.H)), dim3(256), 0, stream>>>(
+        (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, (const T*)p.a, (const T*)p.b,
+        p.h0, p.h0_batch_stride, nullptr, 0, nullptr, nullptr, seq_layout(p, nullptr), states, seg);
+    return hipGetLastError();
+}
+
+// the forward without outputs, storing the state at the start of every segment of `seg` tokens (dense batches)
+hipError_t launch_fwd_recurrent_states(const SeqArgs& p, float* states, int seg, hipStream_t stream) {
+    if (p.N == 128)
+        return p.dtype == RWKV7_DTYPE_BF16  ? launch_states_t<bf16_t, 128>(p, states, seg, stream)
+               : p.dtype == RWKV7_DTYPE_F16 ? launch_states_t<f16_t, 128>(p, states, seg, stream)
+                                            : launch_states_t<float, 128>(p, states, seg, stream);
+    return p.dtype == RWKV7_DTYPE_BF16  ? launch_states_t<bf16_t, 64>(p, states, seg, stream)
+           : p.dtype == RWKV7_DTYPE_F16 ? launch_states_t<f16_t, 64>(p, states, seg, stream)
+                                        : launch_states_t<float, 64>(p, states, seg, stream);
 }
 
 template <typename T>

@@ -74,6 +74,11 @@ hipError_t launch_chunk_items(const SeqLayout& L, void* items, const float* src,
 // chunked bf16 backward; ws must hold bwd_chunk_workspace_bytes(B, T, H) bytes, 256-byte aligned
 size_t bwd_chunk_workspace_bytes(int B, int T, int H, bool varlen = false);
 hipError_t launch_bwd_chunk(const BwdArgs& p, void* ws, hipStream_t stream);
+// float32 recurrent backward for any dtype, K = V = N in {64, 128}, dense batches (p.cu == NULL):
+// ws holds bwd_recurrent_workspace_bytes(B, T, H, N) bytes (segment states, then per-workgroup scratch)
+size_t bwd_recurrent_workspace_bytes(int B, int T, int H, int N);
+hipError_t launch_bwd_recurrent(const BwdArgs& p, int N, void* ws, hipStream_t stream);
+hipError_t launch_fwd_recurrent_states(const SeqArgs& p, float* states, int seg, hipStream_t stream);
 // RWKV6 backward (stateless call, bf16): runs the RWKV7 backward kernels on operands read one token ahead
 // plus an epilogue for the bonus term; du is float32 [H, 64]
 size_t rwkv6_bwd_workspace_bytes(int B, int T, int H);

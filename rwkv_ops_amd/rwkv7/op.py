@@ -33,7 +33,7 @@ import torch
 from . import _lib
 
 HEAD_SIZE = 64
-# K = V = 128 has the decode step and the float32 recurrent forward only (no chunked MFMA kernels, no backward)
+# K = V = 128 has the decode step and the float32 recurrent forward and backward (no chunked MFMA kernels)
 HEAD_SIZES = (64, 128)
 
 __all__ = ["generalized_delta_rule", "rwkv7_decode_step", "HEAD_SIZE"]
@@ -178,6 +178,35 @@ def _(r, w, k, v, a, b, h0, d_o, d_ht):
     return tuple(torch.empty_like(r) for _ in range(6)) + (r.new_empty((B, H, N, N), dtype=torch.float32),)
 
 
+@torch.library.custom_op("rwkv_ops_amd::rwkv7_bwd_recurrent", mutates_args=(), device_types="cuda")
+def rwkv7_bwd_recurrent(r: torch.Tensor, w: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                        a: torch.Tensor, b: torch.Tensor, h0: Optional[torch.Tensor],
+                        d_o: Optional[torch.Tensor], d_ht: Optional[torch.Tensor]
+                        ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
+                                   torch.Tensor, torch.Tensor]:
+    """Gradients of ``rwkv7_fwd`` from the float32 recurrent backward: any of the three dtypes, head size 64
+    or 128; same arguments and results as ``rwkv7_bwd`` (gradients in the dtype of the inputs)."""
+    lib = _lib.load()
+    B, T, H, N = r.shape
+    grads = [torch.empty_like(r) for _ in range(6)]
+    dh0 = torch.empty((B, H, N, N), dtype=torch.float32, device=r.device)
+    with _on_device(r.device):
+        ws_bytes = lib.rwkv7_bwd_recurrent_workspace_bytes(B, T, H, N)
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=r.device)
+        rc = lib.rwkv7_bwd_recurrent(_ptr(r), _ptr(w), _ptr(k), _ptr(v), _ptr(a), _ptr(b),
+                                     _ptr(h0), _h0_stride(h0, B, H), _ptr(d_o), _ptr(d_ht),
+                                     *[_ptr(x) for x in grads], _ptr(dh0),
+                                     B, T, H, N, N, _dtype_code(r.dtype), _ptr(ws), ws_bytes, _stream_ptr(r.device))
+    _lib.check(rc, "rwkv7_bwd_recurrent")
+    return (*grads, dh0)
+
+
+@rwkv7_bwd_recurrent.register_fake
+def _(r, w, k, v, a, b, h0, d_o, d_ht):
+    B, T, H, N = r.shape
+    return tuple(torch.empty_like(r) for _ in range(6)) + (r.new_empty((B, H, N, N), dtype=torch.float32),)
+
+
 def _fwd_setup_context(ctx, inputs, output):
     r, w, k, v, a, b, h0, want_state, state_map = inputs
     ctx.save_for_backward(r, w, k, v, a, b, h0, state_map)   # inputs only: the backward recomputes
@@ -189,15 +218,22 @@ def _fwd_backward(ctx, d_o, d_ht):
     # with a map the backward kernels see the gathered states; dh0 is scattered back below
     h0 = h0_arg if state_map is None else h0_arg.index_select(0, state_map.long())
     dt = r.dtype
-    # The backward kernels are bf16; float32 inputs are rounded to bf16 for the backward only
-    # (the reference's kernel path rounds them for the forward as well, torch_op.py:451-455).
-    cast = (lambda t: t.to(torch.bfloat16)) if dt != torch.bfloat16 else (lambda t: t)
-    d_o_c = None if d_o is None else cast(d_o).contiguous()
     d_ht_c = None
     if ctx.want_state and d_ht is not None and d_ht.numel() > 0:
         d_ht_c = d_ht.to(torch.float32).contiguous()
-    dr, dw, dk, dv, da, db, dh0 = torch.ops.rwkv_ops_amd.rwkv7_bwd(
-        cast(r), cast(w), cast(k), cast(v), cast(a), cast(b), h0, d_o_c, d_ht_c)
+    if dt == torch.float32 or r.shape[-1] != HEAD_SIZE:
+        # float32 calls get float32 gradients, and head size 128 has no chunked backward: both take the
+        # float32 recurrent backward, which reads any of the three dtypes as it is
+        d_o_c = None if d_o is None else d_o.to(dt).contiguous()
+        dr, dw, dk, dv, da, db, dh0 = torch.ops.rwkv_ops_amd.rwkv7_bwd_recurrent(
+            r, w, k, v, a, b, h0, d_o_c, d_ht_c)
+    else:
+        # The chunked backward kernels are bf16; float16 inputs are rounded to bf16 for them, as the reference's
+        # kernel path rounds every input (torch_op.py:451-455).
+        cast = (lambda t: t.to(torch.bfloat16)) if dt != torch.bfloat16 else (lambda t: t)
+        d_o_c = None if d_o is None else cast(d_o).contiguous()
+        dr, dw, dk, dv, da, db, dh0 = torch.ops.rwkv_ops_amd.rwkv7_bwd(
+            cast(r), cast(w), cast(k), cast(v), cast(a), cast(b), h0, d_o_c, d_ht_c)
     g0 = None
     if h0 is not None and ctx.needs_input_grad[6]:
         if state_map is not None:
@@ -449,8 +485,8 @@ def _as_cu_seqlens(cu_seqlens, T: int, device: torch.device) -> torch.Tensor:
 
 def _no_wide_gradients(*tensors) -> None:
     if tensors[0].shape[-1] != HEAD_SIZE and not _direct(*tensors) and not torch.compiler.is_compiling():
-        raise NotImplementedError(f"head size {tensors[0].shape[-1]}: only the forward is built "
-                                  f"(gradients need K = V = {HEAD_SIZE}); call under torch.no_grad()")
+        raise NotImplementedError(f"head size {tensors[0].shape[-1]} with cu_seqlens: only the forward is built "
+                                  f"(packed-sequence gradients need K = V = {HEAD_SIZE}); call under torch.no_grad()")
 
 
 def _check_inputs(r, w, k, v, a, b, initial_state, head_first, mapped=False):
@@ -524,7 +560,6 @@ def generalized_delta_rule(
     h0 = None
     if initial_state is not None:
         h0 = initial_state.to(torch.float32).contiguous()
-    _no_wide_gradients(r_, w_, k_, v_, a_, b_, h0)
     smap = None
     if state_map is not None:
         smap = _as_state_map(state_map, r_.shape[0], h0.shape[0], r_.device)

@@ -1,5 +1,5 @@
 """K = V = 128 (the head size of the reference's own value test, test_script/test_rwkv7_value.py:51): the
-decode step and the float32 recurrent forward, against the CPU oracle (which is written for any head size).
+decode step, the float32 recurrent forward and the float32 recurrent backward, against the CPU oracle (which is written for any head size).
 float32 inputs 1e-4, bf16 inputs 5e-3 relative L2 (the arithmetic is float32 either way; bf16 only rounds o)."""
 import pytest
 import torch
@@ -50,8 +50,31 @@ def test_decode_steps_state_pool_and_packed_sequences(device):
     assert rel_l2(o.reshape(B, T, H, N), o_ref) < 5e-3 and rel_l2(s, s_ref) < 1e-4
 
 
-def test_gradients_are_refused(device):
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 4e-3)])
+def test_gradients_at_the_reference_value_test_shape(device, dtype, tol):
+    """The shape of the reference's own value test (/root/reference/test_script/test_rwkv7_value.py:48-53:
+    T = 128, B = 2, H = 6, head size 128): all seven gradients from the float32 recurrent backward against float32
+    autograd through the oracle on the same rounded inputs.  float32: 1e-4; bf16: the gradients are rounded to
+    bf16 on store (2^-9 per element), nothing else is."""
+    B, T, H = 2, 128, 6
+    xs = make_inputs(B, T, H, N, seed=9200, dtype=dtype)
+    g = torch.Generator().manual_seed(9201)
+    dO = torch.randn(B, T, H, N, generator=g).to(dtype)
+    dS = 0.1 * torch.randn(B, H, N, N, generator=g)
+    ref = orc.gradients(*xs[:6], xs[6], dO, dS)
+    leaves = [x.to(device).requires_grad_(True) for x in xs]
+    o, s = rwkv_ops_amd.generalized_delta_rule(*leaves[:6], initial_state=leaves[6])
+    loss = (o.float() * dO.to(device).float()).sum() + (s * dS.to(device)).sum()
+    got = torch.autograd.grad(loss, leaves)
+    errs = {n: rel_l2(g_, r_) for n, g_, r_ in zip(["dr", "dw", "dk", "dv", "da", "db", "dh0"], got, ref)}
+    print(f"K=128 {dtype}:", " ".join(f"{k}={v:.2e}" for k, v in errs.items()))
+    for name, g_ in zip(errs, got):
+        assert g_.dtype == (torch.float32 if name == "dh0" else dtype)
+        assert errs[name] < (1e-4 if name == "dh0" else tol), (name, errs)
+
+
+def test_packed_gradients_are_refused(device):
     xs = make_inputs(1, 8, 1, N, seed=9200, dtype=torch.bfloat16)
     leaves = [x.to(device).requires_grad_(True) for x in xs[:6]]
-    with pytest.raises(NotImplementedError, match="forward"):
-        rwkv_ops_amd.generalized_delta_rule(*leaves)
+    with pytest.raises(NotImplementedError, match="cu_seqlens"):
+        rwkv_ops_amd.generalized_delta_rule(*leaves, cu_seqlens=[0, 3, 8])
