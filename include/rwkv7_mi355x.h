@@ -46,11 +46,11 @@ extern "C" {
 /* element type of r, w, k, v, a, b, o and the input gradients */
 #define RWKV7_DTYPE_BF16 0
 #define RWKV7_DTYPE_F32  1
-#define RWKV7_DTYPE_F16  2   /* float16: read by the decode step and the float32 recurrent forward only (values are
-                              * widened on load, o is rounded on store).  rwkv7_fwd, rwkv7_fwd_gather and
-                              * rwkv7_fwd_varlen therefore run the recurrent kernel for every T with it; the
-                              * chunked kernels, the backward and the RWKV6 entry points answer
-                              * RWKV7_ERR_UNSUPPORTED.  (The reference's kernel path casts float16 inputs to
+#define RWKV7_DTYPE_F16  2   /* float16: read by the decode step and the float32 recurrent forward and backward
+                              * only (values are widened on load, o and the gradients are rounded on store).
+                              * rwkv7_fwd, rwkv7_fwd_gather and rwkv7_fwd_varlen therefore run the recurrent kernel
+                              * for every T with it; the chunked kernels, rwkv7_bwd and the RWKV6 entry points
+                              * answer RWKV7_ERR_UNSUPPORTED.  (The reference's kernel path casts float16 inputs to
                               * bfloat16, torch_op.py:451-455; callers who want that speed for long T do the
                               * same and pass RWKV7_DTYPE_BF16.) */
 
@@ -85,9 +85,11 @@ const char* rwkv7_status_string(int status);
  * through a 64-token chunk; float32 arithmetic, no workspace used).  Two calls that overlap
  * in time must not share a workspace.
  * K = V = 128 (the head size of /root/reference/test_script/test_rwkv7_value.py:51): accepted by
- * rwkv7_fwd, rwkv7_fwd_gather, rwkv7_fwd_varlen, rwkv7_fwd_recurrent and the two decode-step calls; there
- * are no chunked kernels for it, so T > 1 runs the float32 recurrent kernel for either dtype (no workspace
- * needed; about 1 us per token) and the backward returns RWKV7_ERR_BAD_HEAD_SIZE. */
+ * rwkv7_fwd, rwkv7_fwd_gather, rwkv7_fwd_varlen, rwkv7_fwd_noalloc, rwkv7_fwd_recurrent, the two decode-step
+ * calls and rwkv7_bwd_recurrent.  bf16 with T > 12 runs a chunked MFMA kernel of its own (one workgroup per
+ * (batch, head) walking the chunks with the state in registers; no workspace, ws may be NULL); float32, float16
+ * and T <= 12 run the float32 recurrent kernel (about 1 us per token).  rwkv7_bwd answers
+ * RWKV7_ERR_BAD_HEAD_SIZE for it: its gradients come from rwkv7_bwd_recurrent. */
 size_t rwkv7_fwd_workspace_bytes(int B, int T, int H, int dtype);
 int rwkv7_fwd(const void* r, const void* w, const void* k, const void* v,
               const void* a, const void* b,

@@ -12,7 +12,7 @@ namespace {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// wide_ok: the entry point also has kernels for K = V = 128 (the decode step and the recurrent forward)
+// wide_ok: the entry point also has kernels for K = V = 128
 int check_seq(const void* r, const void* w, const void* k, const void* v, const void* a,
               const void* b, const float* h0, int64_t h0_batch_stride, const void* o,
               const float* ht, int B, int T, int H, int K, int V, int dtype, bool wide_ok = false,
@@ -59,7 +59,7 @@ const char* rwkv7_status_string(int status) {
         case RWKV7_OK: return "ok";
         case RWKV7_ERR_NULL_POINTER: return "a required pointer is NULL";
         case RWKV7_ERR_BAD_DTYPE: return "dtype must be RWKV7_DTYPE_BF16 (0), RWKV7_DTYPE_F32 (1) or RWKV7_DTYPE_F16 (2)";
-        case RWKV7_ERR_BAD_HEAD_SIZE: return "K = V = 64 (every entry point) or 128 (forward and decode step, no chunked kernels) only";
+        case RWKV7_ERR_BAD_HEAD_SIZE: return "K = V = 64 (every entry point) or 128 (forward, decode step and rwkv7_bwd_recurrent) only";
         case RWKV7_ERR_BAD_SHAPE: return "B, T and H must be >= 1 and B*H*ceil(T/64) <= 2^30";
         case RWKV7_ERR_BAD_STRIDE: return "h0_batch_stride must be 0 (broadcast) or H*K*V";
         case RWKV7_ERR_WORKSPACE: return "workspace is NULL, not 256-byte aligned or too small";
@@ -105,6 +105,9 @@ bool use_fused_forward(int B, int H) { return (int64_t)B * H >= 96; }
 // number of sequences: B*H = 2560, T = 2 / 8 / 16 / 32: 17 / 30 / 49 / 89 us against 46 / 46 / 47 / 49 us
 // chunked; B*H = 40: 3.6 / 5.9 / 8.9 / 16 against 10 us.
 constexpr int RECURRENT_MAX_T = 12;
+// K = V = 128 in bf16 beyond that length: the chunked kernel for that head size (one workgroup per sequence and
+// head, state in registers, no workspace)
+bool takes_chunk128(const SeqArgs& p) { return p.N == 128 && p.dtype == RWKV7_DTYPE_BF16 && p.T > RECURRENT_MAX_T; }
 }  // namespace
 
 size_t rwkv7_fwd_workspace_bytes(int B, int T, int H, int dtype) {
@@ -139,6 +142,7 @@ int rwkv7_fwd(const void* r, const void* w, const void* k, const void* v, const 
     if (rc != RWKV7_OK) return rc;
     SeqArgs p = pack(r, w, k, v, a, b, h0, h0_batch_stride, o, ht, B, T, H, dtype, K);
     if (T == 1) return (int)rwkv7::launch_decode(p, static_cast<hipStream_t>(stream));
+    if (takes_chunk128(p)) return (int)rwkv7::launch_fwd_chunk128(p, static_cast<hipStream_t>(stream));
     if (dtype != RWKV7_DTYPE_BF16 || K == 128 || T <= RECURRENT_MAX_T)   // the chunked kernels are K = V = 64 only
         return (int)rwkv7::launch_fwd_recurrent(p, static_cast<hipStream_t>(stream));
     const size_t need = rwkv7_fwd_workspace_bytes(B, T, H, dtype);
@@ -185,6 +189,7 @@ int rwkv7_fwd_noalloc(const void* r, const void* w, const void* k, const void* v
     SeqArgs p = pack(r, w, k, v, a, b, h0, h0_batch_stride, o, ht, B, T, H, dtype, K);
     // the same routing as rwkv7_fwd for the kernels that use no workspace
     if (T == 1) return (int)rwkv7::launch_decode(p, static_cast<hipStream_t>(stream));
+    if (takes_chunk128(p)) return (int)rwkv7::launch_fwd_chunk128(p, static_cast<hipStream_t>(stream));
     if (dtype != RWKV7_DTYPE_BF16 || K == 128 || T <= RECURRENT_MAX_T)
         return (int)rwkv7::launch_fwd_recurrent(p, static_cast<hipStream_t>(stream));
     // Always the one-kernel form: its workspace does not grow with T.
@@ -210,6 +215,7 @@ int rwkv7_fwd_gather(const void* r, const void* w, const void* k, const void* v,
     SeqArgs p = pack(r, w, k, v, a, b, states, (int64_t)H * K * V, o, ht, B, T, H, dtype, K);
     p.h0_map = state_map; p.n_state = n_state;
     if (T == 1) return (int)rwkv7::launch_decode(p, static_cast<hipStream_t>(stream));
+    if (takes_chunk128(p)) return (int)rwkv7::launch_fwd_chunk128(p, static_cast<hipStream_t>(stream));
     if (dtype != RWKV7_DTYPE_BF16 || K == 128 || T <= RECURRENT_MAX_T)
         return (int)rwkv7::launch_fwd_recurrent(p, static_cast<hipStream_t>(stream));
     const size_t need = rwkv7_fwd_workspace_bytes(B, T, H, dtype);
@@ -354,6 +360,7 @@ int rwkv7_fwd_varlen(const void* r, const void* w, const void* k, const void* v,
     if (rc != RWKV7_OK) return rc;
     SeqArgs p = pack(r, w, k, v, a, b, h0, h0_batch_stride, o, ht, n_seq, T_total, H, dtype, K);
     p.cu = cu_seqlens;
+    if (takes_chunk128(p)) return (int)rwkv7::launch_fwd_chunk128(p, static_cast<hipStream_t>(stream));
     if (dtype != RWKV7_DTYPE_BF16 || K == 128)
         return (int)rwkv7::launch_fwd_recurrent(p, static_cast<hipStream_t>(stream));
     const size_t need = rwkv7_fwd_varlen_workspace_bytes(n_seq, T_total, H, dtype);

@@ -48,6 +48,9 @@ hipError_t launch_fwd_fused(const SeqArgs& p, void* ws, hipStream_t stream);
 hipError_t launch_fwd_chunk_summary(const SeqArgs& p, void* ws, hipStream_t stream);
 hipError_t launch_fwd_chunk_scan(const SeqArgs& p, void* ws, hipStream_t stream);
 
+// chunked bf16 forward for K = V = 128 (p.N == 128): no workspace; dense or packed (p.cu), state map honoured
+hipError_t launch_fwd_chunk128(const SeqArgs& p, hipStream_t stream);
+
 struct BwdArgs {
     const void *r, *w, *k, *v, *a, *b;
     const float* h0;          // nullable

@@ -33,7 +33,7 @@ import torch
 from . import _lib
 
 HEAD_SIZE = 64
-# K = V = 128 has the decode step and the float32 recurrent forward and backward (no chunked MFMA kernels)
+# K = V = 128 has the decode step, a chunked bf16 forward of its own and the float32 recurrent forward and backward
 HEAD_SIZES = (64, 128)
 
 __all__ = ["generalized_delta_rule", "rwkv7_decode_step", "HEAD_SIZE"]

@@ -24,8 +24,91 @@ def test_forward_matches_oracle(device, B, T, H, dtype, tol):
     assert o.dtype == dtype and tuple(s.shape) == (B, H, N, N)
     eo, es = rel_l2(o, o_ref), rel_l2(s, s_ref)
     print(f"B={B} T={T} H={H} {dtype}: rel_l2 o={eo:.2e} state={es:.2e}")
-    assert eo < tol and es < min(tol, 1e-4)
+    # bf16 beyond 12 tokens takes the chunked MFMA kernel (bf16 operands: the 5e-3 tolerance holds for the state
+    # too); everything else is float32 arithmetic
+    assert eo < tol and es < (tol if (dtype == torch.bfloat16 and T > 12) else 1e-4)
     assert rel_l2(s, s_ref.transpose(-1, -2)) > 1e-2
+
+
+@pytest.mark.parametrize("B,T,H", [(1, 13, 1), (1, 64, 2), (2, 65, 1), (1, 200, 3), (2, 128, 6), (3, 1000, 2), (1, 4096, 4)])
+def test_chunked_forward_matches_oracle(device, B, T, H):
+    """bf16, K = V = 128, more than 12 tokens: the chunked MFMA kernel for this head size; (2, 128, 6) is the shape
+    of the reference's value test (test_script/test_rwkv7_value.py:48-53).  5e-3 relative L2 on o and the state."""
+    from oracle import native_c
+    xs = make_inputs(B, T, H, N, seed=9300 + T, dtype=torch.bfloat16)
+    with torch.no_grad():
+        o, s = rwkv_ops_amd.generalized_delta_rule(*[x.to(device) for x in xs[:6]], initial_state=xs[6].to(device))
+    o_ref, s_ref = native_c.run(*xs[:6], xs[6])
+    eo, es = rel_l2(o, o_ref), rel_l2(s, s_ref)
+    print(f"K=128 chunked B={B} T={T} H={H}: rel_l2 o={eo:.2e} state={es:.2e}")
+    assert o.dtype == torch.bfloat16 and torch.isfinite(o.float()).all()
+    assert eo < 5e-3 and es < 5e-3, (eo, es)
+    assert rel_l2(s, s_ref.transpose(-1, -2)) > 1e-2
+
+
+@pytest.mark.parametrize("wdist", ["normal", "slow", "mixed"])
+def test_chunked_forward_decay_ranges(device, wdist):
+    """w ~ N(0, 1) (what the reference's smoke test feeds) needs several exponent buckets per chunk."""
+    from oracle import native_c
+    B, T, H = 2, 256, 2
+    xs = list(make_inputs(B, T, H, N, seed=9400, dtype=torch.bfloat16))
+    g = torch.Generator().manual_seed(1)
+    if wdist == "normal":
+        xs[1] = torch.randn(B, T, H, N, generator=g).to(torch.bfloat16)
+    elif wdist == "slow":
+        xs[1] = (-5.0 + torch.randn(B, T, H, N, generator=g)).to(torch.bfloat16)
+    else:
+        xs[1] = (3.0 * torch.randn(B, T, H, N, generator=g) - 1.0).to(torch.bfloat16)
+    with torch.no_grad():
+        o, s = rwkv_ops_amd.generalized_delta_rule(*[x.to(device) for x in xs[:6]], initial_state=xs[6].to(device))
+    o_ref, s_ref = native_c.run(*xs[:6], xs[6])
+    eo, es = rel_l2(o, o_ref), rel_l2(s, s_ref)
+    print(f"K=128 {wdist}: rel_l2 o={eo:.2e} state={es:.2e}")
+    assert torch.isfinite(o.float()).all() and torch.isfinite(s).all()
+    assert eo < 5e-3 and es < 5e-3, (eo, es)
+
+
+def test_chunked_forward_variants(device):
+    """No initial state, a shared one, a state map, padding by w = -1e9, packed sequences: each against the
+    oracle run the plain way."""
+    from oracle import native_c
+    B, T, H = 3, 150, 2
+    xs = make_inputs(B, T, H, N, seed=9500, dtype=torch.bfloat16)
+    d = [x.to(device) for x in xs]
+    with torch.no_grad():
+        o, s = rwkv_ops_amd.generalized_delta_rule(*d[:6])
+        o_ref, s_ref = native_c.run(*xs[:6], None)
+        assert rel_l2(o, o_ref) < 5e-3 and rel_l2(s, s_ref) < 5e-3
+        o, s = rwkv_ops_amd.generalized_delta_rule(*d[:6], initial_state=d[6][:1])
+        o_ref, s_ref = native_c.run(*xs[:6], xs[6][:1])
+        assert rel_l2(o, o_ref) < 5e-3 and rel_l2(s, s_ref) < 5e-3
+        o, s = rwkv_ops_amd.generalized_delta_rule(*d[:6], initial_state=d[6], state_map=[2, 0, 2])
+        o_ref, s_ref = native_c.run(*xs[:6], xs[6][[2, 0, 2]])
+        assert rel_l2(o, o_ref) < 5e-3 and rel_l2(s, s_ref) < 5e-3
+        # the last 40 tokens padded: state untouched by them, outputs zero
+        pad = 40
+        mask = torch.ones(B, T, 1, 1)
+        mask[:, T - pad:] = 0
+        ys = [(xs[i].float() * mask).to(torch.bfloat16) if i != 1 else (xs[1].float() + (1 - mask) * -1e9).to(torch.bfloat16)
+              for i in range(6)]
+        o, s = rwkv_ops_amd.generalized_delta_rule(*[y.to(device) for y in ys], initial_state=d[6])
+        o2, s2 = rwkv_ops_amd.generalized_delta_rule(*[y[:, :T - pad].to(device) for y in ys], initial_state=d[6])
+        assert torch.equal(s, s2) and torch.equal(o[:, :T - pad], o2) and float(o[:, T - pad:].float().abs().max()) == 0.0
+        # packed: lengths 150, 0, 20, 130 in one row of 320 tokens (20 rows behind the last sequence)
+        row = [torch.cat([x[0], x[1]], 0)[None].contiguous() for x in d[:6]]          # [1, 300, H, N]
+        row = [torch.cat([x, x[:, :20]], 1).contiguous() for x in row]                 # [1, 320, ...]
+        cu = [0, 150, 150, 170, 300]
+        h4 = torch.cat([d[6], d[6][:1]], 0)
+        o, s = rwkv_ops_amd.generalized_delta_rule(*row, initial_state=h4, cu_seqlens=cu)
+        for i in range(4):
+            a_, b_ = cu[i], cu[i + 1]
+            if a_ == b_:
+                assert torch.equal(s[i], h4[i])
+                continue
+            o_ref, s_ref = native_c.run(*[x[:, a_:b_].cpu() for x in row], h4[i:i + 1].cpu())
+            tol = 1e-2 if b_ - a_ < 64 else 5e-3
+            assert rel_l2(o[:, a_:b_], o_ref) < tol and rel_l2(s[i:i + 1], s_ref) < tol, i
+        assert float(o[:, 300:].float().abs().max()) == 0.0
 
 
 def test_decode_steps_state_pool_and_packed_sequences(device):
@@ -47,7 +130,8 @@ def test_decode_steps_state_pool_and_packed_sequences(device):
     packed = [x.reshape(1, B * T, H, N) for x in d[:6]]
     with torch.no_grad():
         o, s = rwkv_ops_amd.generalized_delta_rule(*packed, initial_state=d[6], cu_seqlens=[0, T, 2 * T, 3 * T])
-    assert rel_l2(o.reshape(B, T, H, N), o_ref) < 5e-3 and rel_l2(s, s_ref) < 1e-4
+    # (a packed bf16 row of more than 12 tokens takes the chunked kernel: bf16 operands, 5e-3 on the state too)
+    assert rel_l2(o.reshape(B, T, H, N), o_ref) < 5e-3 and rel_l2(s, s_ref) < 5e-3
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 4e-3)])
