@@ -339,6 +339,36 @@ def main():
     f32_bytes = 7 * B * T * H * N * 4 + 2 * B * H * N * N * 4
     del x32, o32
 
+    # float32 gradients at the training shape: the float32 recurrent backward (rwkv7_bwd with float32 tensors)
+    xb32 = [t.float() for t in xb[:6]]
+    d_o32 = d_o.float()
+    g32 = [torch.empty_like(xb32[0]) for _ in range(6)]
+    rws_bytes = lib.rwkv7_bwd_workspace_bytes(Bb, Tb, Hb, 1)
+    rws = torch.empty(rws_bytes, dtype=torch.uint8, device=dev)
+
+    def bwd_f32():
+        rc = lib.rwkv7_bwd(*[ptr(t) for t in xb32], ptr(xb[6]), Hb * N * N, ptr(d_o32), ptr(d_ht),
+                           *[ptr(g) for g in g32], ptr(dh0), Bb, Tb, Hb, N, N, 1, ptr(rws), rws_bytes, stream)
+        assert rc == 0, rc
+
+    ms_bwd_f32, _ = time_gpu(bwd_f32, max(3, args.steps // 40), 1, torch)
+    del xb32, d_o32, g32, rws
+
+    # ------------------------------------------------------------------ head size 128 (bf16, chunked forward)
+    N2, B2, T2, H2 = 128, 8, 4096, 16                       # hidden 2048 as 16 heads of 128
+    x128 = [t.to(dev) for t in make_inputs(B2, T2, H2, N2, seed=1240, dtype=torch.bfloat16)]
+    o128 = torch.empty_like(x128[0])
+    ht128 = torch.empty_like(x128[6])
+
+    def fwd_128():
+        rc = lib.rwkv7_fwd(*[ptr(t) for t in x128[:6]], ptr(x128[6]), H2 * N2 * N2, ptr(o128), ptr(ht128),
+                           B2, T2, H2, N2, N2, 0, None, 0, stream)
+        assert rc == 0, rc
+
+    ms_128, _ = time_gpu(fwd_128, max(10, args.steps // 10), 2, torch)
+    bytes_128 = 7 * B2 * T2 * H2 * N2 * 2 + 2 * B2 * H2 * N2 * N2 * 4
+    del x128, o128, ht128
+
     # ------------------------------------------------------------------ CPU baseline (rank 0, N = 1)
     cpu = None
     if not args.no_cpu:
@@ -457,6 +487,13 @@ def main():
                                 "kernel: 1e-4 parity with the reference's native path)",
                     "ms": ms_f32, "tokens_per_s": B * T / (ms_f32 * 1e-3), "us_per_token": ms_f32 * 1e3 / T,
                     "algorithmic_bytes": f32_bytes, "frac_of_hbm_peak": f32_bytes / (ms_f32 * 1e-3) / HBM_PEAK},
+        "float32_backward": {"workload": f"rwkv7_bwd on float32 tensors (the float32 recurrent backward, forward states "
+                                         f"recomputed inside), B={Bb} T={Tb} H={Hb}, all seven gradients",
+                             "ms": ms_bwd_f32, "us_per_token": ms_bwd_f32 * 1e3 / Tb},
+        "head128": {"workload": f"rwkv7_fwd, K=V=128, B={B2} T={T2} H={H2} bf16 (the chunked kernel for that head size: one "
+                                "workgroup per (batch, head), state in registers), float32 states in and out",
+                    "ms": ms_128, "tokens_per_s": B2 * T2 / (ms_128 * 1e-3), "us_per_chunk": ms_128 * 1e3 / (T2 // 64),
+                    "algorithmic_bytes": bytes_128, "frac_of_hbm_peak": bytes_128 / (ms_128 * 1e-3) / HBM_PEAK},
         "rwkv6": {"workload": f"RWKV6 operator forward (rwkv6_fwd), B={B} T={T} H={H} bf16, float32 states in and out",
                   "ms": ms_rwkv6, "tokens_per_s": B * T / (ms_rwkv6 * 1e-3), "algorithmic_bytes": rwkv6_bytes,
                   "frac_of_hbm_peak": rwkv6_bytes / (ms_rwkv6 * 1e-3) / HBM_PEAK},
