@@ -303,10 +303,11 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         }
     }
     float gl[8], gstep[8], gsum[8];
+    const float vmask = valid ? 1.f : 0.f;     // (times zero rather than a select: no branch around each evaluation)
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
         const float wv = (float)in.W[e];
-        gstep[e] = valid ? fmaxf(-LOG2E * ex2(LOG2E * wv), G_MIN2) : 0.f;     // log2 of exp(-exp(w))
+        gstep[e] = vmask * fmaxf(-LOG2E * ex2(LOG2E * wv), G_MIN2);           // log2 of exp(-exp(w))
         gl[e] = row_inclusive_scan(gstep[e]);
     }
     float* tot = reinterpret_cast<float*>(smem + OFF_TOT);

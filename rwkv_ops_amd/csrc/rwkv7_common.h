@@ -41,12 +41,29 @@ __device__ __forceinline__ int64_t state_row(const int* map, int n_state, int bi
 // one packed row of T tokens in all, sequence bi = rows cu[bi] .. cu[bi + 1] - 1.  What is read from cu is
 // clamped into [0, T] and the end to at least the start, so no value in it can send an access outside the
 // tensors (overlapping or unordered entries give meaningless results, not faults).
+// Division of an index below 2^31 by a divisor that is fixed per launch, as one 64-bit multiply and a shift
+// (the host prepares the multiplier: mul = ceil(2^(31 + sh) / d), sh = ceil(log2 d); exact for every n < 2^31).
+// An integer division by a run-time value costs about 25 scalar instructions on gfx950, and the chunk kernels
+// take three of them per chunk coordinate.
+struct FastDiv { uint32_t mul, sh, d; };
+inline FastDiv make_fast_div(uint32_t d) {
+    FastDiv f;
+    f.d = d; f.sh = 0;
+    while ((1ull << f.sh) < d) ++f.sh;
+    f.mul = (uint32_t)(((1ull << (31 + f.sh)) + d - 1) / d);
+    return f;
+}
+__device__ __forceinline__ int fast_div(int n, const FastDiv& f) {
+    return (int)(((uint64_t)(uint32_t)n * f.mul) >> (31 + f.sh));
+}
+
 struct SeqLayout {
     const int* cu;       // nullable, device memory
     const int* items;    // with cu, chunked kernels only: items[0] = number of chunks over all sequences,
                          // then from items[4] on, in launch order, four ints per chunk: sequence, chunk
                          // within it, first token row and length of the sequence
     int B, T, H;
+    FastDiv dBH, dH;     // division by B * H and by H
 };
 struct SeqSpan { int64_t tok0; int len; };
 

@@ -171,11 +171,11 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
     // of every eighth one was tried: + 1 % at 256 sequences, but twice as slow at 128.)
     // The first workgroup (dispatched first) opens the launch's status record: "not given up", then the tag.
     // A replay of a captured graph repeats the tag, so the flag an earlier replay may have left is taken away here.
-    if (blockIdx.x == 0 && threadIdx.x == 0 && fa.status != nullptr) {
+    if ((blockIdx.x | blockIdx.y | blockIdx.z) == 0 && threadIdx.x == 0 && fa.status != nullptr) {
         __hip_atomic_store(fa.status, fa.tag - 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store(fa.status + 1, fa.tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    const ChunkCoord cc = chunk_coord(L, (int)blockIdx.x);
+    const ChunkCoord cc = chunk_coord_grid(L);
     if (!cc.live) return;              // packed sequences: the grid covers the most chunks there can be
     const int H = L.H, BH = L.B * L.H;
     const int c = cc.c, hi = cc.hi, bi = cc.bi, bh = bi * H + hi;
@@ -212,10 +212,13 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
                 R[0] = R[1] = K[0] = K[1] = V[0] = V[1] = A[0] = A[1] = B[0] = B[1] = z;
             }
         }
+        // (rows past the end: times zero rather than a select, which the compiler turns into a branch around
+        // every one of the sixteen evaluations)
+        const float vmask = valid ? 1.f : 0.f;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             const float wv = (float)W[e >> 3][e & 7];
-            gl[e] = valid ? fmaxf(-LOG2E * ex2(LOG2E * wv), G_MIN) : 0.f;     // log2 of exp(-exp(w))
+            gl[e] = vmask * fmaxf(-LOG2E * ex2(LOG2E * wv), G_MIN);           // log2 of exp(-exp(w))
         }
     }
     float gstep[16];
@@ -1139,6 +1142,7 @@ SeqLayout seq_layout(const SeqArgs& p, const void* ws) {
     SeqLayout L;
     L.cu = p.cu; L.items = p.cu ? static_cast<const int*>(ws) : nullptr;
     L.B = p.B; L.T = p.T; L.H = p.H;
+    L.dBH = make_fast_div((uint32_t)p.B * (uint32_t)p.H); L.dH = make_fast_div((uint32_t)p.H);
     return L;
 }
 
@@ -1177,7 +1181,17 @@ hipError_t launch_summary_kernel(const SeqArgs& p, int64_t nchunks, bf16_t* qt, 
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(chunk_summary_kernel<MODE, V6>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if (e != hipSuccess) return e;
-    chunk_summary_kernel<MODE, V6><<<dim3((unsigned)nchunks), dim3(256), LDS_BYTES, stream>>>(
+    // (head, sequence, chunk) or, packed, (head, item) as grid coordinates where they fit: no integer divisions in
+    // the kernel; the dispatch order is the same as that of the linear index
+    dim3 grid((unsigned)nchunks);
+    const int64_t per_head = nchunks / p.H;
+    if (p.cu == nullptr) {
+        const int64_t nt = per_head / p.B;
+        if (p.B <= 65535 && nt <= 65535) grid = dim3((unsigned)p.H, (unsigned)p.B, (unsigned)nt);
+    } else if (per_head <= 65535) {
+        grid = dim3((unsigned)p.H, (unsigned)per_head);
+    }
+    chunk_summary_kernel<MODE, V6><<<grid, dim3(256), LDS_BYTES, stream>>>(
         (const bf16_t*)p.r, (const bf16_t*)p.w, (const bf16_t*)p.k, (const bf16_t*)p.v,
         (const bf16_t*)p.a, (const bf16_t*)p.b, qt, pp, oi, qc, eg, L, fa);
     return hipGetLastError();

@@ -129,8 +129,8 @@ void chunk128_fwd_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restrict
         auto decays = [&](bool valid, float (&gl)[16], float (&gstep)[16], float (&gsum)[16]) {
     #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const float gs = fmaxf(-LOG2E * ex2(LOG2E * (float)W[e >> 3][e & 7]), G_MIN2);     // log2 of exp(-exp(w))
-                gstep[e] = valid ? gs : 0.f;
+                // log2 of exp(-exp(w)); rows past the end: times zero (a select becomes a branch around each evaluation)
+                gstep[e] = (valid ? 1.f : 0.f) * fmaxf(-LOG2E * ex2(LOG2E * (float)W[e >> 3][e & 7]), G_MIN2);
                 gl[e] = row_inclusive_scan(gstep[e]);
                 if ((e & 3) == 3) __builtin_amdgcn_sched_barrier(0);      // (keeps the sixteen evaluations from being interleaved)
             }

@@ -33,14 +33,40 @@ template <int PACKED = -1>
 __device__ __forceinline__ ChunkCoord chunk_coord(const SeqLayout& L, int n) {
     ChunkCoord q;
     if (PACKED == 0 || (PACKED < 0 && L.cu == nullptr)) {
-        const int BH = L.B * L.H, bh = n % BH;
-        q.c = n / BH; q.hi = bh % L.H; q.bi = bh / L.H;
+        q.c = fast_div(n, L.dBH);
+        const int bh = n - q.c * (L.B * L.H);
+        q.bi = fast_div(bh, L.dH); q.hi = bh - q.bi * L.H;
         q.tok0 = (int64_t)q.bi * L.T; q.len = L.T; q.nt = (L.T + CHUNK_TOKENS - 1) / CHUNK_TOKENS;
         q.rec = n; q.live = true;
         return q;
     }
-    const int item = n / L.H;
-    q.hi = n % L.H;
+    const int item = fast_div(n, L.dH);
+    q.hi = n - item * L.H;
+    q.live = item < load_table(L.items);
+    if (!q.live) { q.tok0 = 0; q.rec = 0; q.bi = 0; q.c = 0; q.len = 0; q.nt = 0; return q; }
+    const int4_t e = load_table4(L.items + 4 + 4 * item);
+    q.bi = e.x; q.c = e.y;
+    const SeqSpan sp = SeqSpan{(int64_t)e.z, e.w};
+    q.tok0 = sp.tok0; q.len = sp.len; q.nt = (sp.len + CHUNK_TOKENS - 1) / CHUNK_TOKENS;
+    q.rec = chunk_record(L, sp, q.bi, q.hi, q.c);
+    return q;
+}
+
+// The same for a kernel launched over a two- or three-dimensional grid, which spares the integer divisions:
+// dense, grid (H, B, chunks): workgroup (x, y, z) = (head, sequence, chunk); packed, grid (H, items): (head, item).
+// Workgroups are dispatched in the order of x + X (y + Y z), which is the launch index n of chunk_coord.  A
+// one-dimensional grid (sizes beyond the 65535 that y and z can hold) falls back to chunk_coord.
+__device__ __forceinline__ ChunkCoord chunk_coord_grid(const SeqLayout& L) {
+    if (gridDim.y == 1 && gridDim.z == 1) return chunk_coord(L, (int)blockIdx.x);
+    ChunkCoord q;
+    q.hi = (int)blockIdx.x;
+    if (L.cu == nullptr) {
+        q.bi = (int)blockIdx.y; q.c = (int)blockIdx.z;
+        q.tok0 = (int64_t)q.bi * L.T; q.len = L.T; q.nt = (L.T + CHUNK_TOKENS - 1) / CHUNK_TOKENS;
+        q.rec = ((int64_t)q.c * L.B + q.bi) * L.H + q.hi; q.live = true;
+        return q;
+    }
+    const int item = (int)blockIdx.y;
     q.live = item < load_table(L.items);
     if (!q.live) { q.tok0 = 0; q.rec = 0; q.bi = 0; q.c = 0; q.len = 0; q.nt = 0; return q; }
     const int4_t e = load_table4(L.items + 4 + 4 * item);
