@@ -200,7 +200,8 @@ constexpr int S_STAGE0 = SLOT(4), S_STAGE1 = SLOT(6), S_STAGE2 = SLOT(11); // fl
 constexpr int OFF_TOT = SLOT(15);            // float [4][64]  sub-block totals of the log decay
 constexpr int OFF_DI = OFF_TOT + 1024;       // 4 inverted diagonal blocks, bf16 16x16
 constexpr int OFF_RED = OFF_DI + 2048;       // float [4][64] + [4][64] reduction scratch
-constexpr int BWD_LDS_BYTES = OFF_RED + 2048;
+constexpr int OFF_EGB = OFF_RED + 2048;      // float [64]: decay of the whole chunk per key channel
+constexpr int BWD_LDS_BYTES = OFF_EGB + 256;
 constexpr int LDZ = 68;                      // row stride (floats) of a staging tile [channel][token]
 
 // Eight waves: wave (w, hf) = (id & 3, id >> 2).  In the load layout (prologue and epilogue) a lane owns
@@ -391,18 +392,31 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     auto get_row = [&](int off) {
         return *reinterpret_cast<const bf16x8_t*>(smem + off + (t_local * LDT + ch0) * 2);
     };
-    // kg, bg rows (bucket-free: exponent G - gi <= 0), kept for the tiles written later and for dG
+    // Several buckets: kg, bg rows (bucket-free: exponent G - gi <= 0), kept for the tiles written later and for dG.
+    // One bucket: kg = k~ diag(e^G) and bg = b~ diag(e^G) with k~, b~ already in their tiles, so the chunk decay is
+    // folded into dh' instead (DECAY_IN_DH): every product with kg or bg takes k~ or b~ against e^G dh', the
+    // gradients of kg and bg come out times e^G, which is what dk, db and dG need of them, and no kg / bg tile,
+    // no e^{G - gi} and no barrier around their slot is left.
+    constexpr bool DECAY_IN_DH = !GENERAL;
     bf16x8_t KG, BG;
     {
         bf16x8_t Qp, Ap, Kp, Bp;
         bucket_operands(0, R, K, A, B, Qp, Ap, Kp, Bp);
         put_operands(Qp, Ap, Kp, Bp);
         put_row(S_V, V); put_row(S_DO, DO);
+        if constexpr (DECAY_IN_DH) {
+            if (w == 0 && x == 0) {
+                float4_t* e4 = reinterpret_cast<float4_t*>(reinterpret_cast<float*>(smem + OFF_EGB) + ch0);
+                e4[0] = float4_t{ex2(gsum[0]), ex2(gsum[1]), ex2(gsum[2]), ex2(gsum[3])};
+                e4[1] = float4_t{ex2(gsum[4]), ex2(gsum[5]), ex2(gsum[6]), ex2(gsum[7])};
+            }
+        } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float tail = ex2(gsum[e] - gl[e]);
-            KG[e] = (bf16_t)(raw(K, e) * tail);
-            BG[e] = (bf16_t)(raw(B, e) * tail);
+            for (int e = 0; e < 8; ++e) {
+                const float tail = ex2(gsum[e] - gl[e]);
+                KG[e] = (bf16_t)(raw(K, e) * tail);
+                BG[e] = (bf16_t)(raw(B, e) * tail);
+            }
         }
     }
     __syncthreads();
@@ -581,9 +595,12 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         float dgdec[8];                    // partial over this lane's value column, key rows 16(2hf+m)+4g+e
 #pragma unroll
         for (int m = 0; m < 2; ++m) {
-            tile_store_acc(smem, S_DH, w, 2 * hf + m, lane, dhimg[m]);
+            float4_t dh = dhimg[m];
+            if constexpr (DECAY_IN_DH)
+                dh = dh * *reinterpret_cast<const float4_t*>(reinterpret_cast<const float*>(smem + OFF_EGB) + 16 * (2 * hf + m) + 4 * g);
+            tile_store_acc(smem, S_DH, w, 2 * hf + m, lane, dh);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) dgdec[4 * m + e] = h0img[m][e] * dhimg[m][e];
+            for (int e = 0; e < 4; ++e) dgdec[4 * m + e] = h0img[m][e] * dh[e];      // (DECAY_IN_DH: e^G included)
         }
         // reduce over the 16 value columns of the row, then (later) over the 4 value tiles through LDS
         float* red = reinterpret_cast<float*>(smem + OFF_RED);
@@ -596,7 +613,7 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
                     float4_t{dgdec[4 * m], dgdec[4 * m + 1], dgdec[4 * m + 2], dgdec[4 * m + 3]};
         }
     }
-    put_row(S_BG, BG);
+    if constexpr (!DECAY_IN_DH) put_row(S_BG, BG);
     __syncthreads();
 
     // accumulators that live to the end: rows = tokens, column = channel 16w + x
@@ -613,14 +630,16 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     const FragB DOc = loadB(colsB(S_DO)), DHr = loadB(rowsB(S_DH));
     clear(tmp);
     gemm_ar(tmp, colsA(S_AQB), DOc);
-    gemm_ar(tmp, rowsA(S_BG), DHr);
+    gemm_ar(tmp, rowsA(DECAY_IN_DH ? S_BT : S_BG), DHr);
     store_tile(S_DSA, tmp);
-    __syncthreads();                       // bg is dead: its slot takes kg
-    put_row(S_KG, KG);
-    __syncthreads();
+    if constexpr (!DECAY_IN_DH) {
+        __syncthreads();                   // bg is dead: its slot takes kg
+        put_row(S_KG, KG);
+        __syncthreads();
+    }
     // dV[j][v] = Aqk^T dO + kg dh' (+ Aak^T dY below)
     gemm_ar(acc_v, colsA(S_AQK), DOc);
-    gemm_ar(acc_v, rowsA(S_KG), DHr);
+    gemm_ar(acc_v, rowsA(DECAY_IN_DH ? S_KT : S_KG), DHr);
     __syncthreads();                       // dh' is dead: its slot takes dY
     // dY[j][v] = M^T dSA              -> dY^T[v][j]
     clear(tmp);
@@ -716,24 +735,25 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         stage_get(stg(3), zb); stage_get(stg(4), zbg); stage_get(stg(5), zq); stage_get(stg(6), za);
         float out[8];
         prefetch_next(P4{});
-        float ek[8], et[8];
+        float ek[8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { ek[e] = ex2(-gl[e]); et[e] = ex2(gsum[e] - gl[e]); }
-        // dk = dkt e^{-gi} + dkg e^{G-gi}, dv
+        for (int e = 0; e < 8; ++e) ek[e] = ex2(-gl[e]);
+        // dk = dkt e^{-gi} + dkg e^{G-gi}, dv.  zkg, zbg are the gradients of kg, bg times e^G (the decay went
+        // into dh'): e^G dkg e^{-gi} is the second term, and dkg kg = (e^G dkg) k~.
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            out[e] = zk[e] * ek[e] + zkg[e] * et[e];
+            out[e] = (zk[e] + zkg[e]) * ek[e];
             sall[e] = -zk[e] * (float)Kp[e];
-            dkk[e] = zkg[e] * (float)KG[e];
+            dkk[e] = zkg[e] * (float)Kp[e];
         }
         store_rows(dk_, pack_rows(out));
         store_rows(dv_, pack_rows(zv));
         // db, dr
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            out[e] = zb[e] * ek[e] + zbg[e] * et[e];
+            out[e] = (zb[e] + zbg[e]) * ek[e];
             sall[e] -= zb[e] * (float)Bp[e];
-            dkk[e] += zbg[e] * (float)BG[e];
+            dkk[e] += zbg[e] * (float)Bp[e];
         }
         store_rows(db_, pack_rows(out));
 #pragma unroll
@@ -877,7 +897,7 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         }
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-            dg[e] = sfx[e] + later[e] - dge[e] + dGs[e] + ex2(gsum[e]) * dec[e];
+            dg[e] = sfx[e] + later[e] - dge[e] + dGs[e] + (DECAY_IN_DH ? dec[e] : ex2(gsum[e]) * dec[e]);
     }
     {
         float dwv[8];
