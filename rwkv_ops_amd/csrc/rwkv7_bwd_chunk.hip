@@ -197,6 +197,11 @@ constexpr int S_SA = SLOT(12);                                             // SA
 constexpr int S_BG = SLOT(13), S_KG = SLOT(13), S_DAAK = SLOT(13);         // bg -> kg -> dAak
 constexpr int S_DSA = SLOT(14), S_DAAB = SLOT(14);                         // dSA^T -> dAab
 constexpr int S_STAGE0 = SLOT(4), S_STAGE1 = SLOT(6), S_STAGE2 = SLOT(11); // float staging, 2 slots each
+// The one-bucket kernel has no bg / kg tile, which leaves two slots free from the start: h0^T and dh'^T get slots of
+// their own and are written in the prologue, and every later tile lands in a slot whose previous tenant's last read
+// lies behind a barrier that is needed anyway.  Its plan where it differs from the one above:
+//   9: Aab -> dSA^T -> dAqk    7: Aqb -> dAak    13: h0^T    14: dh'^T -> dAab    11: Y^T -> dY^T
+constexpr int S1_H0 = SLOT(13), S1_DH = SLOT(14), S1_DSA = SLOT(9), S1_DAAK = SLOT(7);
 constexpr int OFF_TOT = SLOT(15);            // float [4][64]  sub-block totals of the log decay
 constexpr int OFF_DI = OFF_TOT + 1024;       // 4 inverted diagonal blocks, bf16 16x16
 constexpr int OFF_RED = OFF_DI + 2048;       // float [4][64] + [4][64] reduction scratch
@@ -398,6 +403,9 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     // gradients of kg and bg come out times e^G, which is what dk, db and dG need of them, and no kg / bg tile,
     // no e^{G - gi} and no barrier around their slot is left.
     constexpr bool DECAY_IN_DH = !GENERAL;
+    // (slots of the tiles whose place depends on the plan)
+    constexpr int T_H0 = DECAY_IN_DH ? S1_H0 : S_H0, T_DH = DECAY_IN_DH ? S1_DH : S_DH;
+    constexpr int T_DSA = DECAY_IN_DH ? S1_DSA : S_DSA, T_DAAK = DECAY_IN_DH ? S1_DAAK : S_DAAK;
     bf16x8_t KG, BG;
     {
         bf16x8_t Qp, Ap, Kp, Bp;
@@ -405,6 +413,9 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         put_operands(Qp, Ap, Kp, Bp);
         put_row(S_V, V); put_row(S_DO, DO);
         if constexpr (DECAY_IN_DH) {
+            // h0^T tile [v][c] from the float image; wave = (value tile w, key tiles 2hf, 2hf + 1)
+#pragma unroll
+            for (int m = 0; m < 2; ++m) tile_store_acc(smem, T_H0, w, 2 * hf + m, lane, h0img[m]);
             if (w == 0 && x == 0) {
                 float4_t* e4 = reinterpret_cast<float4_t*>(reinterpret_cast<float*>(smem + OFF_EGB) + ch0);
                 e4[0] = float4_t{ex2(gsum[0]), ex2(gsum[1]), ex2(gsum[2]), ex2(gsum[3])};
@@ -420,6 +431,31 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         }
     }
     __syncthreads();
+
+    // ---- dh'^T tile [v][c]; the decay part of dG needs  sum_v h0 dh'  in float32
+    auto adjoint_tile = [&]() {
+        float dgdec[8];                    // partial over this lane's value column, key rows 16(2hf+m)+4g+e
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+            float4_t dh = dhimg[m];
+            if constexpr (DECAY_IN_DH)
+                dh = dh * *reinterpret_cast<const float4_t*>(reinterpret_cast<const float*>(smem + OFF_EGB) + 16 * (2 * hf + m) + 4 * g);
+            tile_store_acc(smem, T_DH, w, 2 * hf + m, lane, dh);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dgdec[4 * m + e] = h0img[m][e] * dh[e];      // (DECAY_IN_DH: e^G included)
+        }
+        // reduce over the 16 value columns of the row, then (later) over the 4 value tiles through LDS
+        float* red = reinterpret_cast<float*>(smem + OFF_RED);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dgdec[i] = row_inclusive_suffix_scan(dgdec[i]);   // lane x = 0: the row's sum
+        if (x == 0) {
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+                *reinterpret_cast<float4_t*>(red + w * 64 + 16 * (2 * hf + m) + 4 * g) =
+                    float4_t{dgdec[4 * m], dgdec[4 * m + 1], dgdec[4 * m + 2], dgdec[4 * m + 3]};
+        }
+    };
+    if constexpr (DECAY_IN_DH) adjoint_tile();     // its slot is free from the start, e^G is there since the barrier
 
     // ---- G1: block row w (rows j, column i = 16w + x) of Aqk, Aqb (waves hf = 0) and of Aak, Aab
     // (waves hf = 1), bucket by bucket
@@ -526,12 +562,15 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
             }
         }
     }
-    __syncthreads();                       // Aab is dead from here: its slot takes h0
-
-    // ---- h0^T tile [v][c] from the float image; wave = (value tile w, key tiles 2hf, 2hf + 1)
+    if constexpr (!DECAY_IN_DH) {
+        __syncthreads();                   // Aab is dead from here: its slot takes h0
+        // ---- h0^T tile [v][c] from the float image; wave = (value tile w, key tiles 2hf, 2hf + 1)
 #pragma unroll
-    for (int m = 0; m < 2; ++m) tile_store_acc(smem, S_H0, w, 2 * hf + m, lane, h0img[m]);
-    __syncthreads();
+        for (int m = 0; m < 2; ++m) tile_store_acc(smem, T_H0, w, 2 * hf + m, lane, h0img[m]);
+        __syncthreads();
+    }
+    // (one bucket: h0 has been in its tile since the prologue, so Y needs nothing of the M^T phase and the waves
+    // that do not take part in it start here; the barrier behind Y publishes M^T as well)
 
     // generic product: acc[m] += sum_s A(2hf + m, s) * B(s): this wave's two row tiles of its 16 columns
     auto gemm = [&](float4_t (&acc)[2], auto&& Af, auto&& Bf) {
@@ -580,7 +619,7 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     float4_t tmp[2];
     // Y[j][v] = ag h0 + Aak V        -> Y^T[v][j]
     clear(tmp);
-    gemm(tmp, rowsA(S_AG), rowsB(S_H0));
+    gemm(tmp, rowsA(S_AG), rowsB(T_H0));
     gemm(tmp, rowsA(S_AAK), colsB(S_V));
     store_tile(S_Y, tmp);
     __syncthreads();
@@ -588,50 +627,30 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     clear(tmp);
     gemm(tmp, colsA(S_MT), rowsB(S_Y));
     store_tile(S_SA, tmp);
-    __syncthreads();                       // Y is dead: its slot takes dh'
+    __syncthreads();                       // SA is there; Y is dead (general plan: its slot takes dh')
 
-    // ---- dh'^T tile [v][c]; the decay part of dG needs  sum_v h0 dh'  in float32
-    {
-        float dgdec[8];                    // partial over this lane's value column, key rows 16(2hf+m)+4g+e
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-            float4_t dh = dhimg[m];
-            if constexpr (DECAY_IN_DH)
-                dh = dh * *reinterpret_cast<const float4_t*>(reinterpret_cast<const float*>(smem + OFF_EGB) + 16 * (2 * hf + m) + 4 * g);
-            tile_store_acc(smem, S_DH, w, 2 * hf + m, lane, dh);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) dgdec[4 * m + e] = h0img[m][e] * dh[e];      // (DECAY_IN_DH: e^G included)
-        }
-        // reduce over the 16 value columns of the row, then (later) over the 4 value tiles through LDS
-        float* red = reinterpret_cast<float*>(smem + OFF_RED);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) dgdec[i] = row_inclusive_suffix_scan(dgdec[i]);   // lane x = 0: the row's sum
-        if (x == 0) {
-#pragma unroll
-            for (int m = 0; m < 2; ++m)
-                *reinterpret_cast<float4_t*>(red + w * 64 + 16 * (2 * hf + m) + 4 * g) =
-                    float4_t{dgdec[4 * m], dgdec[4 * m + 1], dgdec[4 * m + 2], dgdec[4 * m + 3]};
-        }
+    if constexpr (!DECAY_IN_DH) adjoint_tile();
+    if constexpr (!DECAY_IN_DH) {
+        put_row(S_BG, BG);
+        __syncthreads();
     }
-    if constexpr (!DECAY_IN_DH) put_row(S_BG, BG);
-    __syncthreads();
 
     // accumulators that live to the end: rows = tokens, column = channel 16w + x
     float4_t acc_q[2], acc_a[2], acc_kg[2], acc_bg[2], acc_v[2];
     clear(acc_q); clear(acc_a); clear(acc_kg); clear(acc_bg); clear(acc_v);
     // dkg[j][c] = V dh'^T ;  dbg[j][c] = SA dh'^T ;  dqg_h[i][c] = dO h0^T
     {
-        const FragB DHc = loadB(colsB(S_DH));
+        const FragB DHc = loadB(colsB(T_DH));
         gemm_ar(acc_kg, rowsA(S_V), DHc);
         gemm_ar(acc_bg, colsA(S_SA), DHc);
     }
-    gemm(acc_q, rowsA(S_DO), colsB(S_H0));
+    gemm(acc_q, rowsA(S_DO), colsB(T_H0));
     // dSA[j][v] = Aqb^T dO + bg dh'   -> dSA^T[v][j]
-    const FragB DOc = loadB(colsB(S_DO)), DHr = loadB(rowsB(S_DH));
+    const FragB DOc = loadB(colsB(S_DO)), DHr = loadB(rowsB(T_DH));
     clear(tmp);
     gemm_ar(tmp, colsA(S_AQB), DOc);
     gemm_ar(tmp, rowsA(DECAY_IN_DH ? S_BT : S_BG), DHr);
-    store_tile(S_DSA, tmp);
+    store_tile(T_DSA, tmp);
     if constexpr (!DECAY_IN_DH) {
         __syncthreads();                   // bg is dead: its slot takes kg
         put_row(S_KG, KG);
@@ -640,15 +659,15 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     // dV[j][v] = Aqk^T dO + kg dh' (+ Aak^T dY below)
     gemm_ar(acc_v, colsA(S_AQK), DOc);
     gemm_ar(acc_v, rowsA(DECAY_IN_DH ? S_KT : S_KG), DHr);
-    __syncthreads();                       // dh' is dead: its slot takes dY
+    __syncthreads();                       // dSA is there (general plan: dh' is dead, its slot takes dY)
     // dY[j][v] = M^T dSA              -> dY^T[v][j]
     clear(tmp);
-    gemm(tmp, rowsA(S_MT), rowsB(S_DSA));
+    gemm(tmp, rowsA(S_MT), rowsB(T_DSA));
     store_tile(S_DY, tmp);
     __syncthreads();                       // M^T, dSA and kg are dead
     gemm(acc_v, colsA(S_AAK), rowsB(S_DY));
-    gemm(acc_a, colsA(S_DY), colsB(S_H0));         // dag_h[i][c] = dY h0^T
-    __syncthreads();                       // h0 is dead: its slot takes dAqk
+    gemm(acc_a, colsA(S_DY), colsB(T_H0));         // dag_h[i][c] = dY h0^T
+    if constexpr (!DECAY_IN_DH) __syncthreads();   // h0 is dead: its slot takes dAqk (one bucket: dSA's, dead since dY)
 
     prefetch_next(P1{});   // the next chunk's inputs land while the last products and the epilogue run
     // ---- dA matrices as tiles [i][j] (column tile w = token tile i; rows of the product are j).  Their
@@ -672,7 +691,7 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         const FragA SAc = loadA(colsA(S_SA));
         clear(d); gemm_rr(d, SAc, DOr); masked_store(S_DAQB, d, false);   // dAqb[i][j] = sum_v SA[j][v] dO[i][v]
         const FragB DYc = loadB(colsB(S_DY));
-        clear(d); gemm_rr(d, Vr, DYc);  masked_store(S_DAAK, d, true);    // dAak[i][j] = sum_v V[j][v] dY[i][v]
+        clear(d); gemm_rr(d, Vr, DYc);  masked_store(T_DAAK, d, true);    // dAak[i][j] = sum_v V[j][v] dY[i][v]
         clear(d); gemm_rr(d, SAc, DYc); masked_store(S_DAAB, d, true);    // dAab[i][j] = sum_v SA[j][v] dY[i][v]
     }
     __syncthreads();
@@ -712,13 +731,13 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         clear(acc_k); clear(acc_b);
         {
             const FragB KTc = loadB(colsB(S_KT));
-            gemm_ar(acc_q, rowsA(S_DAQK), KTc); gemm_ar(acc_a, rowsA(S_DAAK), KTc);
+            gemm_ar(acc_q, rowsA(S_DAQK), KTc); gemm_ar(acc_a, rowsA(T_DAAK), KTc);
             const FragB BTc = loadB(colsB(S_BT));
             gemm_ar(acc_q, rowsA(S_DAQB), BTc); gemm_ar(acc_a, rowsA(S_DAAB), BTc);
             const FragB QGc = loadB(colsB(S_QG));
             gemm_ar(acc_k, colsA(S_DAQK), QGc); gemm_ar(acc_b, colsA(S_DAQB), QGc);
             const FragB AGc = loadB(colsB(S_AG));
-            gemm_ar(acc_k, colsA(S_DAAK), AGc); gemm_ar(acc_b, colsA(S_DAAB), AGc);
+            gemm_ar(acc_k, colsA(T_DAAK), AGc); gemm_ar(acc_b, colsA(S_DAAB), AGc);
         }
         // this lane's pieces of the bucket-0 operands, back from their tiles
         const bf16x8_t Qp = get_row(S_QG), Ap = get_row(S_AG), Kp = get_row(S_KT), Bp = get_row(S_BT);
