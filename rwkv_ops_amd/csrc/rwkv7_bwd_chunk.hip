@@ -704,14 +704,18 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     float* st0 = reinterpret_cast<float*>(smem + S_STAGE0);
     float* st1 = reinterpret_cast<float*>(smem + S_STAGE1);
     float* st2 = reinterpret_cast<float*>(smem + S_STAGE2);
+    // Staging tiles [channel][token] with the tokens of channel ch rotated by 16 (ch / 8): the four lane groups
+    // of a reading wave (channels 8 apart, same tokens) would otherwise all land on the same sixteen banks.
     auto stage_put = [&](float* st, const float4_t (&acc)[2]) {     // [channel 16w+x][token 16mt+4g..]
+        const int rot = 16 * (2 * w + (x >> 3));
 #pragma unroll
         for (int m = 0; m < 2; ++m)
-            *reinterpret_cast<float4_t*>(st + (16 * w + x) * LDZ + 16 * (2 * hf + m) + 4 * g) = acc[m];
+            *reinterpret_cast<float4_t*>(st + (16 * w + x) * LDZ + ((16 * (2 * hf + m) + 4 * g + rot) & 63)) = acc[m];
     };
     auto stage_get = [&](const float* st, float (&z)[8]) {           // this lane's token, its 8 channels
+        const int tr = (t_local + 16 * g) & 63;                      // (ch0 + e) / 8 = 4 hf + g for every e
 #pragma unroll
-        for (int e = 0; e < 8; ++e) z[e] = st[(ch0 + e) * LDZ + t_local];
+        for (int e = 0; e < 8; ++e) z[e] = st[(ch0 + e) * LDZ + tr];
     };
     auto pack_rows = [&](const float (&val)[8]) {
         bf16x8_t o;
