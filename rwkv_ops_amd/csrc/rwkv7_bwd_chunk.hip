@@ -289,6 +289,13 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     const int ch0 = 32 * hf + 8 * g;          // first of this lane's eight channels in the load layout
     const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 
+    // Waits until the next chunk's inputs have landed: a use that the compiler must honour.  Not under the condition of
+    // the requests themselves: the compiler does not see that the two conditions agree, and a path with requests but
+    // without this wait would keep them "in flight" up to the loop's back edge.
+    auto collect_next = [&]() {
+        asm volatile("" :: "v"(next.R), "v"(next.W), "v"(next.K), "v"(next.V), "v"(next.A), "v"(next.B), "v"(next.DO),
+                     "v"(next.h0img[0]), "v"(next.h0img[1]), "v"(next.dhimg[0]), "v"(next.dhimg[1]));
+    };
     auto prefetch_next = [&](auto part) {
         if (n_next >= 0)
             load_chunk_inputs<decltype(part)::value, PACKED>(next, n_next, lane, r_, w_, k_, v_, a_, b_, dO_, hs, dhs, L);
@@ -352,6 +359,7 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         if (npass > 1) {
             if (threadIdx.x == 0) list[1 + atomicAdd(list, 1u)] = (unsigned)n;
             prefetch_next(PALL{});
+            collect_next();                // (so that no path reaches the loop's back edge with requests in flight)
             return;
         }
     }
@@ -734,18 +742,42 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         float4_t acc_k[2], acc_b[2];
         clear(acc_k); clear(acc_b);
         {
+            // Eight products, software-pipelined by hand: the fragments of the next product are requested before the
+            // MFMAs of the current one are issued (the fences keep the compiler from sinking each read next to its
+            // use, where every MFMA would wait out an LDS round trip).
             const FragB KTc = loadB(colsB(S_KT));
-            gemm_ar(acc_q, rowsA(S_DAQK), KTc); gemm_ar(acc_a, rowsA(T_DAAK), KTc);
+            FragA f0 = loadA(rowsA(S_DAQK));
+            FragA f1 = loadA(rowsA(T_DAAK));
+            __builtin_amdgcn_sched_barrier(0);
+            gemm_rr(acc_q, f0, KTc);
             const FragB BTc = loadB(colsB(S_BT));
-            gemm_ar(acc_q, rowsA(S_DAQB), BTc); gemm_ar(acc_a, rowsA(S_DAAB), BTc);
+            f0 = loadA(rowsA(S_DAQB));
+            __builtin_amdgcn_sched_barrier(0);
+            gemm_rr(acc_a, f1, KTc);
+            f1 = loadA(rowsA(S_DAAB));
+            __builtin_amdgcn_sched_barrier(0);
+            gemm_rr(acc_q, f0, BTc);
             const FragB QGc = loadB(colsB(S_QG));
-            gemm_ar(acc_k, colsA(S_DAQK), QGc); gemm_ar(acc_b, colsA(S_DAQB), QGc);
+            f0 = loadA(colsA(S_DAQK));
+            __builtin_amdgcn_sched_barrier(0);
+            gemm_rr(acc_a, f1, BTc);
+            f1 = loadA(colsA(S_DAQB));
+            __builtin_amdgcn_sched_barrier(0);
+            gemm_rr(acc_k, f0, QGc);
             const FragB AGc = loadB(colsB(S_AG));
-            gemm_ar(acc_k, colsA(T_DAAK), AGc); gemm_ar(acc_b, colsA(S_DAAB), AGc);
+            f0 = loadA(colsA(T_DAAK));
+            __builtin_amdgcn_sched_barrier(0);
+            gemm_rr(acc_b, f1, QGc);
+            f1 = loadA(colsA(S_DAAB));
+            __builtin_amdgcn_sched_barrier(0);
+            gemm_rr(acc_k, f0, AGc);
+            __builtin_amdgcn_sched_barrier(0);
+            gemm_rr(acc_b, f1, AGc);
         }
         // this lane's pieces of the bucket-0 operands, back from their tiles
         const bf16x8_t Qp = get_row(S_QG), Ap = get_row(S_AG), Kp = get_row(S_KT), Bp = get_row(S_BT);
         prefetch_next(P3{});
+        prefetch_next(P4{});
         // Every tile is dead now, so all seven accumulator sets change layout in one round: float
         // tiles [channel][token] over the whole tile area, one barrier before and one after.
         __syncthreads();
@@ -757,7 +789,11 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         stage_get(stg(0), zk); stage_get(stg(1), zkg); stage_get(stg(2), zv);
         stage_get(stg(3), zb); stage_get(stg(4), zbg); stage_get(stg(5), zq); stage_get(stg(6), za);
         float out[8];
-        prefetch_next(P4{});
+        // Every request for the next chunk's inputs is collected HERE, before the first store below.  On gfx9 loads and
+        // stores share one in-flight counter and may complete out of order, so with both kinds outstanding the only wait
+        // the compiler can emit for a loaded register is "everything, stores included": left to the loop's back edge, that
+        // wait exposed the full latency of the six output stores once per chunk (12 % of the call).
+        collect_next();
         float ek[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) ek[e] = ex2(-gl[e]);
@@ -950,6 +986,11 @@ __global__ __launch_bounds__(512, 1) void chunk_bwd_kernel(RWKV7_BWD_PARAMS) {
     if (n >= total) return;
     ChunkInputs cur;
     load_chunk_inputs<0x7ffu, PACKED>(cur, n, (int)(threadIdx.x & 63), r_, w_, k_, v_, a_, b_, dO_, hs, dhs, L);
+    // The first chunk's inputs are waited for in front of the loop: with requests in flight at the loop's entry and
+    // stores in flight at its back edge, the compiler has to wait for "everything" at the loop's top, which on the
+    // back edge means the previous chunk's output stores (see chunk_bwd_body).
+    asm volatile("" :: "v"(cur.R), "v"(cur.W), "v"(cur.K), "v"(cur.V), "v"(cur.A), "v"(cur.B), "v"(cur.DO),
+                 "v"(cur.h0img[0]), "v"(cur.h0img[1]), "v"(cur.dhimg[0]), "v"(cur.dhimg[1]));
     while (true) {
         // the lane id is made opaque per iteration so that per-lane addresses are recomputed where they
         // are used instead of being hoisted out of the loop and kept in registers
