@@ -300,10 +300,15 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         if (n_next >= 0)
             load_chunk_inputs<decltype(part)::value, PACKED>(next, n_next, lane, r_, w_, k_, v_, a_, b_, dO_, hs, dhs, L);
     };
+    // Six small groups, each issued in a phase of its own: two groups in one phase cost 3 % of the call (a wave sits at
+    // the issue stage until the memory pipeline has taken its requests), and none in the phases of the inverse and of
+    // M^T, whose waves are the critical path.
     using P1 = std::integral_constant<unsigned, 0x00fu>;      // the two float images
-    using P2 = std::integral_constant<unsigned, 0x070u>;      // w, r, k
-    using P3 = std::integral_constant<unsigned, 0x380u>;      // v, a, b
-    using P4 = std::integral_constant<unsigned, 0x400u>;      // dO
+    using P2 = std::integral_constant<unsigned, 0x030u>;      // w, r
+    using P3 = std::integral_constant<unsigned, 0x040u>;      // k
+    using P4 = std::integral_constant<unsigned, 0x180u>;      // v, a
+    using P5 = std::integral_constant<unsigned, 0x200u>;      // b
+    using P6 = std::integral_constant<unsigned, 0x400u>;      // dO
     using PALL = std::integral_constant<unsigned, 0x7ffu>;
     const float4_t h0img[2] = {in.h0img[0], in.h0img[1]}, dhimg[2] = {in.dhimg[0], in.dhimg[1]};
 
@@ -464,6 +469,9 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         }
     };
     if constexpr (DECAY_IN_DH) adjoint_tile();     // its slot is free from the start, e^G is there since the barrier
+    // The next chunk's inputs are requested from here on, a few at a time: this chunk's copies are dead since the
+    // prologue, so the requests cost no registers, and they have landed long before they are collected.
+    prefetch_next(P1{});
 
     // ---- G1: block row w (rows j, column i = 16w + x) of Aqk, Aqb (waves hf = 0) and of Aak, Aab
     // (waves hf = 1), bucket by bucket
@@ -643,6 +651,7 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         __syncthreads();
     }
 
+    prefetch_next(P2{});
     // accumulators that live to the end: rows = tokens, column = channel 16w + x
     float4_t acc_q[2], acc_a[2], acc_kg[2], acc_bg[2], acc_v[2];
     clear(acc_q); clear(acc_a); clear(acc_kg); clear(acc_bg); clear(acc_v);
@@ -653,6 +662,7 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         gemm_ar(acc_bg, colsA(S_SA), DHc);
     }
     gemm(acc_q, rowsA(S_DO), colsB(T_H0));
+    prefetch_next(P3{});
     // dSA[j][v] = Aqb^T dO + bg dh'   -> dSA^T[v][j]
     const FragB DOc = loadB(colsB(S_DO)), DHr = loadB(rowsB(T_DH));
     clear(tmp);
@@ -673,11 +683,12 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     gemm(tmp, rowsA(S_MT), rowsB(T_DSA));
     store_tile(S_DY, tmp);
     __syncthreads();                       // M^T, dSA and kg are dead
+    prefetch_next(P4{});
     gemm(acc_v, colsA(S_AAK), rowsB(S_DY));
     gemm(acc_a, colsA(S_DY), colsB(T_H0));         // dag_h[i][c] = dY h0^T
     if constexpr (!DECAY_IN_DH) __syncthreads();   // h0 is dead: its slot takes dAqk (one bucket: dSA's, dead since dY)
 
-    prefetch_next(P1{});   // the next chunk's inputs land while the last products and the epilogue run
+    prefetch_next(P5{});
     // ---- dA matrices as tiles [i][j] (column tile w = token tile i; rows of the product are j).  Their
     // slots (h0, M^T, kg, dSA) are dead since the last barrier, so each is stored as soon as it is masked.
     {
@@ -704,7 +715,7 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     }
     __syncthreads();
 
-    prefetch_next(P2{});
+    prefetch_next(P6{});
     // ---- the decay-weighted products and the epilogue in the load layout.
     // dgi / dge are formed from the SAME bf16-rounded operands the products used (z qg - z kt - ...), not
     // from dr r - dk k - db b: the pair terms then cancel exactly in the suffix sum instead of leaving
@@ -776,8 +787,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
         }
         // this lane's pieces of the bucket-0 operands, back from their tiles
         const bf16x8_t Qp = get_row(S_QG), Ap = get_row(S_AG), Kp = get_row(S_KT), Bp = get_row(S_BT);
-        prefetch_next(P3{});
-        prefetch_next(P4{});
         // Every tile is dead now, so all seven accumulator sets change layout in one round: float
         // tiles [channel][token] over the whole tile area, one barrier before and one after.
         __syncthreads();
