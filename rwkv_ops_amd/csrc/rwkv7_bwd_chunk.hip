@@ -747,6 +747,9 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
     };
     // sall = dgi + dge (the suffix-scan input), dge, and dkk = dkg kg + dbg bg (for dG)
     float sall[8], dge[8], dkk[8];
+    // (one bucket: the six output stores are spread over the epilogue and the reductions behind it: stores issued
+    // back to back hold the wave at the issue stage until the memory pipeline has taken them)
+    bf16x8_t late_db, late_dr, late_da;
     if constexpr (!GENERAL) {
         // Common case, one decay bucket: every output is final after one staging round and is stored
         // at once, so only sall / dge / dkk stay live.
@@ -815,7 +818,6 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
             dkk[e] = zkg[e] * (float)Kp[e];
         }
         store_rows(dk_, pack_rows(out));
-        store_rows(dv_, pack_rows(zv));
         // db, dr
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -823,10 +825,11 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
             sall[e] -= zb[e] * (float)Bp[e];
             dkk[e] += zbg[e] * (float)Bp[e];
         }
-        store_rows(db_, pack_rows(out));
+        late_db = pack_rows(out);
+        store_rows(dv_, pack_rows(zv));
 #pragma unroll
         for (int e = 0; e < 8; ++e) { out[e] = zq[e] * ex2(gl[e]); sall[e] += zq[e] * (float)Qp[e]; }
-        store_rows(dr_, pack_rows(out));
+        late_dr = pack_rows(out);
         // da
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -834,7 +837,8 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
             dge[e] = za[e] * (float)Ap[e];
             sall[e] += dge[e] - dkk[e];
         }
-        store_rows(da_, pack_rows(out));
+        late_da = pack_rows(out);
+        store_rows(db_, late_db);
     } else {
         // Several decay buckets (strong decays): one pass of the products per bucket, each with its own
         // exponent offset, accumulated in registers.
@@ -936,6 +940,7 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
             sfx[e] = row_inclusive_suffix_scan(sall[e]);            // over this wave's 16 tokens
             dkk[e] = row_inclusive_suffix_scan(dkk[e]);             // lane x = 0: sum over the wave's 16 tokens
         }
+        if constexpr (!GENERAL) store_rows(dr_, late_dr);
         float* totw = reinterpret_cast<float*>(smem + OFF_TOT);     // [4 token tiles][64]: tile totals of dgi+dge
         if (x == 0) {                                               // token 0 of the tile holds the tile totals
             float4_t* t4 = reinterpret_cast<float4_t*>(totw + w * 64 + ch0);
@@ -944,6 +949,7 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
             r4[0] = float4_t{dkk[0], dkk[1], dkk[2], dkk[3]}; r4[1] = float4_t{dkk[4], dkk[5], dkk[6], dkk[7]};
         }
         __syncthreads();
+        if constexpr (!GENERAL) store_rows(da_, late_da);
         float later[8], dGs[8], dec[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) { later[e] = 0.f; dGs[e] = 0.f; dec[e] = 0.f; }
