@@ -99,19 +99,28 @@ void chunk128_fwd_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restrict
     }
 
     bf16x8_t R[2], W[2], K[2], V[2], A[2], B[2];
-    auto load_chunk = [&](int c, int ln) {
+    // part: bit 0 = w, r; bit 1 = k, v; bit 2 = a, b.  Inside the loop a chunk's inputs are requested in these three
+    // groups, each behind a different product: a wave that issues all twelve requests at once sits at the issue stage
+    // until the memory pipeline has taken them.
+    auto load_chunk = [&](int c, int ln, int part) {
         const int t = c * CH + 16 * w + (ln & 15);
         const int c0 = 64 * hf + 8 * (ln >> 4), c1 = c0 + 32;
         // rows past the sequence's end (last chunk only) are read from the last valid row and zeroed by the consumer
         const int64_t row = ((sp.tok0 + (t < T ? t : T - 1)) * H + hi) * N;
-        R[0] = *reinterpret_cast<const bf16x8_t*>(r_ + row + c0); R[1] = *reinterpret_cast<const bf16x8_t*>(r_ + row + c1);
-        W[0] = *reinterpret_cast<const bf16x8_t*>(w_ + row + c0); W[1] = *reinterpret_cast<const bf16x8_t*>(w_ + row + c1);
-        K[0] = *reinterpret_cast<const bf16x8_t*>(k_ + row + c0); K[1] = *reinterpret_cast<const bf16x8_t*>(k_ + row + c1);
-        V[0] = *reinterpret_cast<const bf16x8_t*>(v_ + row + c0); V[1] = *reinterpret_cast<const bf16x8_t*>(v_ + row + c1);
-        A[0] = *reinterpret_cast<const bf16x8_t*>(a_ + row + c0); A[1] = *reinterpret_cast<const bf16x8_t*>(a_ + row + c1);
-        B[0] = *reinterpret_cast<const bf16x8_t*>(b_ + row + c0); B[1] = *reinterpret_cast<const bf16x8_t*>(b_ + row + c1);
+        if (part & 1) {
+            W[0] = *reinterpret_cast<const bf16x8_t*>(w_ + row + c0); W[1] = *reinterpret_cast<const bf16x8_t*>(w_ + row + c1);
+            R[0] = *reinterpret_cast<const bf16x8_t*>(r_ + row + c0); R[1] = *reinterpret_cast<const bf16x8_t*>(r_ + row + c1);
+        }
+        if (part & 2) {
+            K[0] = *reinterpret_cast<const bf16x8_t*>(k_ + row + c0); K[1] = *reinterpret_cast<const bf16x8_t*>(k_ + row + c1);
+            V[0] = *reinterpret_cast<const bf16x8_t*>(v_ + row + c0); V[1] = *reinterpret_cast<const bf16x8_t*>(v_ + row + c1);
+        }
+        if (part & 4) {
+            A[0] = *reinterpret_cast<const bf16x8_t*>(a_ + row + c0); A[1] = *reinterpret_cast<const bf16x8_t*>(a_ + row + c1);
+            B[0] = *reinterpret_cast<const bf16x8_t*>(b_ + row + c0); B[1] = *reinterpret_cast<const bf16x8_t*>(b_ + row + c1);
+        }
     };
-    if (NT > 0) load_chunk(0, (int)(threadIdx.x & 63));
+    if (NT > 0) load_chunk(0, (int)(threadIdx.x & 63), 7);
     for (int c = 0; c < NT; ++c) {
         // The lane id is made opaque per chunk, so that the per-lane addresses are formed where they are used
         // instead of being hoisted out of the loop and kept in (spilled) registers.
@@ -248,7 +257,7 @@ void chunk128_fwd_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restrict
                 dst[1] = float4_t{dv[4], dv[5], dv[6], dv[7]};
             }
             __syncthreads();
-            if (c + 1 < NT) load_chunk(c + 1, lane);
+            if (c + 1 < NT) load_chunk(c + 1, lane, 7);
             const int nt = T - c * CH < CH ? T - c * CH : CH;
             for (int tt = 0; tt < nt; ++tt) {
                 float4_t sa4 = zero4;          // partial sums over this lane's rows, tile by tile
@@ -401,6 +410,7 @@ void chunk128_fwd_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restrict
             __builtin_amdgcn_sched_barrier(0);
         }
         const bf16x8_t Ys[2] = {pack_sigma(y[0], y[1]), pack_sigma(y[2], y[3])};
+        if (c + 1 < NT) load_chunk(c + 1, lane, 1);        // the next chunk's inputs travel from here on
         __builtin_amdgcn_sched_barrier(0);
         // SA[i][v] = M Y
 #pragma unroll
@@ -411,6 +421,7 @@ void chunk128_fwd_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restrict
             y[it] = acc;
         }
         const bf16x8_t Us[2] = {pack_sigma(y[0], y[1]), pack_sigma(y[2], y[3])};
+        if (c + 1 < NT) load_chunk(c + 1, lane, 2);
         __builtin_amdgcn_sched_barrier(0);
         // O[i][v] = qg h + Aqk V + Aqb SA  -> O^T tile [value][token]
 #pragma unroll
@@ -431,8 +442,7 @@ void chunk128_fwd_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restrict
             __builtin_amdgcn_sched_barrier(0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        // the next chunk's inputs travel while the state is updated and the outputs leave
-        if (c + 1 < NT) load_chunk(c + 1, lane);
+        if (c + 1 < NT) load_chunk(c + 1, lane, 4);
         // h'[c][v] = e^G h + kg^T V + bg^T SA
         {
             const float* eg = reinterpret_cast<const float*>(smem + OFF_EG);
