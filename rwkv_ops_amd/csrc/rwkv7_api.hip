@@ -108,6 +108,9 @@ constexpr int RECURRENT_MAX_T = 12;
 // K = V = 128 in bf16 beyond that length: the chunked kernel for that head size (one workgroup per sequence and
 // head, state in registers, no workspace)
 bool takes_chunk128(const SeqArgs& p) { return p.N == 128 && p.dtype == RWKV7_DTYPE_BF16 && p.T > RECURRENT_MAX_T; }
+// float32 tensors at K = V = 64 beyond that length: the chunked float32 kernel (16-token chunks on the float32 matrix
+// cores, state in registers, no workspace)
+bool takes_chunk_f32(const SeqArgs& p) { return p.N == 64 && p.dtype == RWKV7_DTYPE_F32 && p.T > RECURRENT_MAX_T; }
 }  // namespace
 
 size_t rwkv7_fwd_workspace_bytes(int B, int T, int H, int dtype) {
@@ -143,6 +146,7 @@ int rwkv7_fwd(const void* r, const void* w, const void* k, const void* v, const 
     SeqArgs p = pack(r, w, k, v, a, b, h0, h0_batch_stride, o, ht, B, T, H, dtype, K);
     if (T == 1) return (int)rwkv7::launch_decode(p, static_cast<hipStream_t>(stream));
     if (takes_chunk128(p)) return (int)rwkv7::launch_fwd_chunk128(p, static_cast<hipStream_t>(stream));
+    if (takes_chunk_f32(p)) return (int)rwkv7::launch_fwd_chunk_f32(p, static_cast<hipStream_t>(stream));
     if (dtype != RWKV7_DTYPE_BF16 || K == 128 || T <= RECURRENT_MAX_T)   // the chunked kernels are K = V = 64 only
         return (int)rwkv7::launch_fwd_recurrent(p, static_cast<hipStream_t>(stream));
     const size_t need = rwkv7_fwd_workspace_bytes(B, T, H, dtype);
@@ -190,6 +194,7 @@ int rwkv7_fwd_noalloc(const void* r, const void* w, const void* k, const void* v
     // the same routing as rwkv7_fwd for the kernels that use no workspace
     if (T == 1) return (int)rwkv7::launch_decode(p, static_cast<hipStream_t>(stream));
     if (takes_chunk128(p)) return (int)rwkv7::launch_fwd_chunk128(p, static_cast<hipStream_t>(stream));
+    if (takes_chunk_f32(p)) return (int)rwkv7::launch_fwd_chunk_f32(p, static_cast<hipStream_t>(stream));
     if (dtype != RWKV7_DTYPE_BF16 || K == 128 || T <= RECURRENT_MAX_T)
         return (int)rwkv7::launch_fwd_recurrent(p, static_cast<hipStream_t>(stream));
     // Always the one-kernel form: its workspace does not grow with T.
@@ -216,6 +221,7 @@ int rwkv7_fwd_gather(const void* r, const void* w, const void* k, const void* v,
     p.h0_map = state_map; p.n_state = n_state;
     if (T == 1) return (int)rwkv7::launch_decode(p, static_cast<hipStream_t>(stream));
     if (takes_chunk128(p)) return (int)rwkv7::launch_fwd_chunk128(p, static_cast<hipStream_t>(stream));
+    if (takes_chunk_f32(p)) return (int)rwkv7::launch_fwd_chunk_f32(p, static_cast<hipStream_t>(stream));
     if (dtype != RWKV7_DTYPE_BF16 || K == 128 || T <= RECURRENT_MAX_T)
         return (int)rwkv7::launch_fwd_recurrent(p, static_cast<hipStream_t>(stream));
     const size_t need = rwkv7_fwd_workspace_bytes(B, T, H, dtype);
@@ -361,6 +367,7 @@ int rwkv7_fwd_varlen(const void* r, const void* w, const void* k, const void* v,
     SeqArgs p = pack(r, w, k, v, a, b, h0, h0_batch_stride, o, ht, n_seq, T_total, H, dtype, K);
     p.cu = cu_seqlens;
     if (takes_chunk128(p)) return (int)rwkv7::launch_fwd_chunk128(p, static_cast<hipStream_t>(stream));
+    if (takes_chunk_f32(p)) return (int)rwkv7::launch_fwd_chunk_f32(p, static_cast<hipStream_t>(stream));
     if (dtype != RWKV7_DTYPE_BF16 || K == 128)
         return (int)rwkv7::launch_fwd_recurrent(p, static_cast<hipStream_t>(stream));
     const size_t need = rwkv7_fwd_varlen_workspace_bytes(n_seq, T_total, H, dtype);

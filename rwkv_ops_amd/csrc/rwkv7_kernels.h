@@ -51,6 +51,10 @@ hipError_t launch_fwd_chunk_scan(const SeqArgs& p, void* ws, hipStream_t stream)
 // chunked bf16 forward for K = V = 128 (p.N == 128): no workspace; dense or packed (p.cu), state map honoured
 hipError_t launch_fwd_chunk128(const SeqArgs& p, hipStream_t stream);
 
+// chunked float32 forward (float32 tensors, K = V = 64) on the float32 matrix cores: no workspace; dense or packed
+// (p.cu), state map honoured
+hipError_t launch_fwd_chunk_f32(const SeqArgs& p, hipStream_t stream);
+
 struct BwdArgs {
     const void *r, *w, *k, *v, *a, *b;
     const float* h0;          // nullable
