@@ -483,10 +483,15 @@ def main():
                           "frac_of_hbm_peak": long_bytes / (ms_long * 1e-3) / HBM_PEAK,
                           "chunk_summary_kernel_ms": ms_long_summary, "chunk_scan_vsplit_kernel_ms": ms_long_scan,
                           "scan_us_per_chunk": ms_long_scan * 1e3 / (Tl // 64)},
-        "float32": {"workload": f"generalized_delta_rule on float32 inputs, B={B} T={T} H={H} (the float32 recurrent "
-                                "kernel: 1e-4 parity with the reference's native path)",
+        "float32": {"workload": f"generalized_delta_rule on float32 inputs, B={B} T={T} H={H} (the chunked float32 "
+                                "kernel on the float32 matrix cores: 1e-4 parity with the reference's native path, "
+                                "measured 3e-7)",
                     "ms": ms_f32, "tokens_per_s": B * T / (ms_f32 * 1e-3), "us_per_token": ms_f32 * 1e3 / T,
-                    "algorithmic_bytes": f32_bytes, "frac_of_hbm_peak": f32_bytes / (ms_f32 * 1e-3) / HBM_PEAK},
+                    "algorithmic_bytes": f32_bytes, "frac_of_hbm_peak": f32_bytes / (ms_f32 * 1e-3) / HBM_PEAK,
+                    # executed on the matrix cores per 16-token chunk and (batch, head): 4 x 80 instructions by the
+                    # consumer waves, 96 by the producers, 2048 flops each (v_mfma_f32_16x16x4_f32)
+                    "mfma_f32_executed_tflops": (B * H * ((T + 15) // 16) * 416 * 2048) / (ms_f32 * 1e-3) / 1e12,
+                    "mfma_f32_frac_of_peak": (B * H * ((T + 15) // 16) * 416 * 2048) / (ms_f32 * 1e-3) / 157.3e12},
         "float32_backward": {"workload": f"rwkv7_bwd on float32 tensors (the float32 recurrent backward, forward states "
                                          f"recomputed inside), B={Bb} T={Tb} H={Hb}, all seven gradients",
                              "ms": ms_bwd_f32, "us_per_token": ms_bwd_f32 * 1e3 / Tb},

@@ -79,16 +79,18 @@ const char* rwkv7_status_string(int status);
  * bf16 runs the fused chunked MFMA kernel (one workgroup per 64-token chunk; the
  * state travels from chunk to chunk through the workspace) and needs a workspace of
  * rwkv7_fwd_workspace_bytes() (a few MB: two state slots and four counters per
- * (batch, head)); f32 runs the float32 recurrent kernel and needs none (ws may be
- * NULL).  T == 1 takes the decode kernel for both types, and 2 <= T <= 12 the recurrent
- * kernel (a handful of tokens is faster one at a time with the state in registers than
- * through a 64-token chunk; float32 arithmetic, no workspace used).  Two calls that overlap
+ * (batch, head)); f32 runs the chunked float32 kernel (16-token chunks on the float32
+ * matrix cores, one workgroup per (batch, head) with the state in registers; float32
+ * arithmetic throughout, the accuracy of the reference's native loop) and needs none (ws
+ * may be NULL).  T == 1 takes the decode kernel for both types, and 2 <= T <= 12 the
+ * recurrent kernel (a handful of tokens is faster one at a time with the state in registers
+ * than through a chunk; float32 arithmetic, no workspace used).  Two calls that overlap
  * in time must not share a workspace.
  * K = V = 128 (the head size of /root/reference/test_script/test_rwkv7_value.py:51): accepted by
  * rwkv7_fwd, rwkv7_fwd_gather, rwkv7_fwd_varlen, rwkv7_fwd_noalloc, rwkv7_fwd_recurrent, the two decode-step
  * calls and rwkv7_bwd_recurrent.  bf16 with T > 12 runs a chunked MFMA kernel of its own (one workgroup per
  * (batch, head) walking the chunks with the state in registers; no workspace, ws may be NULL); float32, float16
- * and T <= 12 run the float32 recurrent kernel (about 1 us per token).  rwkv7_bwd answers
+ * and T <= 12 run the float32 recurrent kernel at this head size (about 1 us per token).  rwkv7_bwd answers
  * RWKV7_ERR_BAD_HEAD_SIZE for it: its gradients come from rwkv7_bwd_recurrent. */
 size_t rwkv7_fwd_workspace_bytes(int B, int T, int H, int dtype);
 int rwkv7_fwd(const void* r, const void* w, const void* k, const void* v,
@@ -267,8 +269,8 @@ int rwkv7_bwd_varlen(const void* r, const void* w, const void* k, const void* v,
 
 /* The float32 recurrent kernel for either dtype (inputs are widened on load):
  * the arithmetic of native_keras_op.py:85,87 one token at a time with the state
- * in registers.  Slow; the accurate path for float32 inputs and an on-device
- * cross-check for the chunked kernels. */
+ * in registers.  Slow; what float16 tensors, head size 128 in float32 and sequences of at most 12 tokens
+ * run, and an on-device cross-check for the chunked kernels. */
 int rwkv7_fwd_recurrent(const void* r, const void* w, const void* k, const void* v,
                         const void* a, const void* b,
                         const float* h0, int64_t h0_batch_stride,
