@@ -317,51 +317,54 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
         const float4_t MT = *reinterpret_cast<const float4_t*>(smem + F_BOX + 3 * 1024 + lane * 16);
         // Vg[e] = V[token 4 g + e][16 w + x]: R of V restricted to this wave's columns
         const float4_t Vg = *reinterpret_cast<const float4_t*>(smem + F_VT + ((16 * w + x) * LDC + 4 * g) * 4);
-        // R(Y): Y[j][v] = ag h + Aak V
-        float4_t Y = zero4;
+        // R(Y): Y[j][v] = ag h + Aak V, and the part of O that does not need SA, two independent chains of matrix
+        // instructions issued alternately (an instruction that accumulates onto the previous one's result waits for it).
+        // R(O^T): O^T[v][i] = h^T qg^T + V^T Aqk^T + SA^T Aqb^T -- the operands of O with A and B exchanged, so that
+        // a lane ends up with four consecutive values of ONE token and stores them as 16 bytes
+        float4_t Y = zero4, OT = zero4;
 #pragma unroll
         for (int ct = 0; ct < 4; ++ct) {
             const float4_t af = tile4(smem, F_AG, x, 16 * ct + 4 * g);
+            const float4_t qf = tile4(smem, F_QG, x, 16 * ct + 4 * g);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) Y = mfma_f32(af[e], h[ct][e], Y);
+            for (int e = 0; e < 4; ++e) {
+                Y = mfma_f32(af[e], h[ct][e], Y);
+                OT = mfma_f32(h[ct][e], qf[e], OT);
+            }
         }
 #pragma unroll
-        for (int e = 0; e < 4; ++e) Y = mfma_f32(AakT[e], Vg[e], Y);
+        for (int e = 0; e < 4; ++e) {
+            Y = mfma_f32(AakT[e], Vg[e], Y);
+            OT = mfma_f32(Vg[e], AqkT[e], OT);
+        }
         // R(SA): SA = M Y
         float4_t SA = zero4;
 #pragma unroll
         for (int e = 0; e < 4; ++e) SA = mfma_f32(MT[e], Y[e], SA);
-        // R(O^T): O^T[v][i] = h^T qg^T + V^T Aqk^T + SA^T Aqb^T -- the operands of O with A and B exchanged, so that
-        // a lane ends up with four consecutive values of ONE token and stores them as 16 bytes
-        float4_t OT = zero4;
-#pragma unroll
-        for (int ct = 0; ct < 4; ++ct) {
-            const float4_t qf = tile4(smem, F_QG, x, 16 * ct + 4 * g);
-#pragma unroll
-            for (int e = 0; e < 4; ++e) OT = mfma_f32(h[ct][e], qf[e], OT);
-        }
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            OT = mfma_f32(Vg[e], AqkT[e], OT);
-            OT = mfma_f32(SA[e], AqbT[e], OT);
-        }
-        if (valid) *reinterpret_cast<float4_t*>(o_ + ((sp.tok0 + c * C16 + x) * H + hi) * NH + 16 * w + 4 * g) = OT;
         // h'[c][v] = e^G h + kg^T V + bg^T SA: the A operand is kg[token 4 g + e][channel 16 ct + x], a row of kg^T
+        // (the four tiles and the last of O are five independent chains: one instruction of each in turn; the part
+        // that does not need SA first)
         {
             const float* eg = reinterpret_cast<const float*>(smem + F_EG);
+            float4_t kgf[4], bgf[4];
 #pragma unroll
             for (int ct = 0; ct < 4; ++ct) {
-                float4_t acc = *reinterpret_cast<const float4_t*>(eg + 16 * ct + 4 * g) * h[ct];
-                const float4_t kgf = *reinterpret_cast<const float4_t*>(smem + F_KGT + ((16 * ct + x) * LDC + 4 * g) * 4);
-                const float4_t bgf = *reinterpret_cast<const float4_t*>(smem + F_BGT + ((16 * ct + x) * LDC + 4 * g) * 4);
+                h[ct] = *reinterpret_cast<const float4_t*>(eg + 16 * ct + 4 * g) * h[ct];
+                kgf[ct] = *reinterpret_cast<const float4_t*>(smem + F_KGT + ((16 * ct + x) * LDC + 4 * g) * 4);
+                bgf[ct] = *reinterpret_cast<const float4_t*>(smem + F_BGT + ((16 * ct + x) * LDC + 4 * g) * 4);
+            }
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    acc = mfma_f32(kgf[e], Vg[e], acc);
-                    acc = mfma_f32(bgf[e], SA[e], acc);
-                }
-                h[ct] = acc;
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int ct = 0; ct < 4; ++ct) h[ct] = mfma_f32(kgf[ct][e], Vg[e], h[ct]);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                OT = mfma_f32(SA[e], AqbT[e], OT);
+#pragma unroll
+                for (int ct = 0; ct < 4; ++ct) h[ct] = mfma_f32(bgf[ct][e], SA[e], h[ct]);
             }
         }
+        if (valid) *reinterpret_cast<float4_t*>(o_ + ((sp.tok0 + c * C16 + x) * H + hi) * NH + 16 * w + 4 * g) = OT;
         __syncthreads();
     }
     if (ht != nullptr) {
