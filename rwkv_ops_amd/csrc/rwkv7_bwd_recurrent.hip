@@ -301,7 +301,9 @@ hipError_t launch_bwd_recurrent(const BwdArgs& p, int N, void* ws, hipStream_t s
     f.r = p.r; f.w = p.w; f.k = p.k; f.v = p.v; f.a = p.a; f.b = p.b;
     f.h0 = p.h0; f.h0_batch_stride = p.h0 ? p.h0_batch_stride : 0;
     f.B = p.B; f.T = p.T; f.H = p.H; f.N = N; f.dtype = p.dtype;
-    hipError_t e = launch_fwd_recurrent_states(f, ckpt, seg, stream);
+    // (float32 tensors at head size 64 beyond a dozen tokens: the chunked float32 forward, otherwise the recurrent one)
+    hipError_t e = (N == 64 && p.dtype == RWKV7_DTYPE_F32 && p.T > 12) ? launch_fwd_chunk_f32_states(f, ckpt, seg, stream)
+                                                                      : launch_fwd_recurrent_states(f, ckpt, seg, stream);
     if (e != hipSuccess) return e;
     if (N == 128)
         return p.dtype == RWKV7_DTYPE_BF16  ? launch_bwd_rec_t<bf16_t, 128>(p, ckpt, scratch, stream)

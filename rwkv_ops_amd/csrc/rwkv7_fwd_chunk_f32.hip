@@ -87,8 +87,11 @@ __global__ __launch_bounds__(768)
 void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restrict__ w_, const float* __restrict__ k_,
                             const float* __restrict__ v_, const float* __restrict__ a_, const float* __restrict__ b_,
                             const float* __restrict__ h0, int64_t h0_batch_stride, const int* __restrict__ h0_map,
-                            int n_state, float* __restrict__ o_, float* __restrict__ ht, SeqLayout L)
+                            int n_state, float* __restrict__ o_, float* __restrict__ ht, SeqLayout L,
+                            float* __restrict__ seg_states, int seg)
 {
+    // seg_states (dense batches): the state BEFORE token t is stored for every t that is a multiple of `seg` (a
+    // multiple of 16), [workgroup][t / seg][64][64]: what the recurrent backward restarts from.  o_ may then be NULL.
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_all[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int w = wave & 3;                    // consumers: value columns 16 w .. + 15; producers: channels 16 w .. + 15
@@ -280,6 +283,13 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
         const int x = lane & 15, g = lane >> 4;
         const unsigned char* smem = smem_all + (c % 3) * BUF_BYTES;
         const bool valid = c * C16 + x < T;
+        if (seg_states != nullptr && (c * C16) % seg == 0) {
+            float* dst = seg_states + ((int64_t)bh * ((T + seg - 1) / seg) + (c * C16) / seg) * (NH * NH) + 16 * w + x;
+#pragma unroll
+            for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dst[(16 * ct + 4 * g + e) * NH] = h[ct][e];
+        }
         bool strong;
         {
             const int* fl = reinterpret_cast<const int*>(smem + F_FLAG);
@@ -306,7 +316,7 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
                 float ov = (o4[0] + o4[1]) + (o4[2] + o4[3]);
                 ov += __shfl_xor(ov, 16, 64);
                 ov += __shfl_xor(ov, 32, 64);
-                if (g == 0) o_[((sp.tok0 + c * C16 + tt) * H + hi) * NH + 16 * w + x] = ov;
+                if (g == 0 && o_ != nullptr) o_[((sp.tok0 + c * C16 + tt) * H + hi) * NH + 16 * w + x] = ov;
             }
             __syncthreads();
             continue;
@@ -364,7 +374,8 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
                 for (int ct = 0; ct < 4; ++ct) h[ct] = mfma_f32(bgf[ct][e], SA[e], h[ct]);
             }
         }
-        if (valid) *reinterpret_cast<float4_t*>(o_ + ((sp.tok0 + c * C16 + x) * H + hi) * NH + 16 * w + 4 * g) = OT;
+        if (valid && o_ != nullptr)
+            *reinterpret_cast<float4_t*>(o_ + ((sp.tok0 + c * C16 + x) * H + hi) * NH + 16 * w + 4 * g) = OT;
         __syncthreads();
     }
     if (ht != nullptr) {
@@ -387,7 +398,20 @@ hipError_t launch_fwd_chunk_f32(const SeqArgs& p, hipStream_t stream) {
     if (e != hipSuccess) return e;
     chunk16_f32_fwd_kernel<<<dim3((unsigned)(p.B * p.H)), dim3(768), LDS_F32_BYTES, stream>>>(
         (const float*)p.r, (const float*)p.w, (const float*)p.k, (const float*)p.v, (const float*)p.a,
-        (const float*)p.b, p.h0, p.h0_batch_stride, p.h0_map, p.n_state, (float*)p.o, p.ht, seq_layout(p, nullptr));
+        (const float*)p.b, p.h0, p.h0_batch_stride, p.h0_map, p.n_state, (float*)p.o, p.ht, seq_layout(p, nullptr),
+        nullptr, 0);
+    return hipGetLastError();
+}
+
+// the forward without outputs, storing the state at the start of every segment of `seg` tokens (dense batches,
+// float32 tensors, K = V = 64; seg a multiple of 16)
+hipError_t launch_fwd_chunk_f32_states(const SeqArgs& p, float* states, int seg, hipStream_t stream) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(chunk16_f32_fwd_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, LDS_F32_BYTES);
+    if (e != hipSuccess) return e;
+    chunk16_f32_fwd_kernel<<<dim3((unsigned)(p.B * p.H)), dim3(768), LDS_F32_BYTES, stream>>>(
+        (const float*)p.r, (const float*)p.w, (const float*)p.k, (const float*)p.v, (const float*)p.a,
+        (const float*)p.b, p.h0, p.h0_batch_stride, nullptr, 0, nullptr, nullptr, seq_layout(p, nullptr), states, seg);
     return hipGetLastError();
 }
 

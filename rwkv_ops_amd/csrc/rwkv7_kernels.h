@@ -54,6 +54,8 @@ hipError_t launch_fwd_chunk128(const SeqArgs& p, hipStream_t stream);
 // chunked float32 forward (float32 tensors, K = V = 64) on the float32 matrix cores: no workspace; dense or packed
 // (p.cu), state map honoured
 hipError_t launch_fwd_chunk_f32(const SeqArgs& p, hipStream_t stream);
+// the same kernel without outputs, storing the state at the start of every `seg` tokens ([B*H][ceil(T/seg)][64][64])
+hipError_t launch_fwd_chunk_f32_states(const SeqArgs& p, float* states, int seg, hipStream_t stream);
 
 struct BwdArgs {
     const void *r, *w, *k, *v, *a, *b;
