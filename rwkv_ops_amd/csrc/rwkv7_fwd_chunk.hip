@@ -196,8 +196,8 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         // read from the last valid row and zeroed afterwards.
         const int64_t row_ld = valid ? row : ((cc.tok0 + (T - 1)) * H + hi) * HEAD;
         const int c0 = 8 * g, c1 = 32 + 8 * g;
-        R[0] = load_frag_global(r_ + row_ld + c0, true); R[1] = load_frag_global(r_ + row_ld + c1, true);
         W[0] = load_frag_global(w_ + row_ld + c0, true); W[1] = load_frag_global(w_ + row_ld + c1, true);
+        R[0] = load_frag_global(r_ + row_ld + c0, true); R[1] = load_frag_global(r_ + row_ld + c1, true);
         K[0] = load_frag_global(k_ + row_ld + c0, true); K[1] = load_frag_global(k_ + row_ld + c1, true);
         V[0] = load_frag_global(v_ + row_ld + c0, true); V[1] = load_frag_global(v_ + row_ld + c1, true);
         if constexpr (V6) {
