@@ -274,7 +274,9 @@ int rwkv7_fwd_chunk_scan(const float* h0, int64_t h0_batch_stride, void* o, floa
 
 size_t rwkv7_bwd_workspace_bytes(int B, int T, int H, int dtype) {
     if (B < 1 || T < 1 || H < 1) return 0;
-    if (dtype == RWKV7_DTYPE_F32) return rwkv7::bwd_recurrent_workspace_bytes(B, T, H, 64);
+    if (dtype == RWKV7_DTYPE_F32)
+        return T > RECURRENT_MAX_T ? rwkv7::bwd_chunk_f32_workspace_bytes(B, T, H)
+                                   : rwkv7::bwd_recurrent_workspace_bytes(B, T, H, 64);
     if (dtype != RWKV7_DTYPE_BF16) return 0;
     return rwkv7::bwd_chunk_workspace_bytes(B, T, H);
 }
@@ -311,10 +313,28 @@ int rwkv7_bwd(const void* r, const void* w, const void* k, const void* v, const 
               void* dr, void* dw, void* dk, void* dv, void* da, void* db, float* dh0,
               int B, int T, int H, int K, int V, int dtype, void* ws, size_t ws_bytes, void* stream)
 {
-    // float32 gradients come from the float32 recurrent backward (K = V = 64 here; rwkv7_bwd_recurrent takes 128 too)
-    if (dtype == RWKV7_DTYPE_F32 && K == 64 && V == 64)
-        return rwkv7_bwd_recurrent(r, w, k, v, a, b, h0, h0_batch_stride, d_o, d_ht, dr, dw, dk, dv, da, db, dh0,
-                                   B, T, H, K, V, dtype, ws, ws_bytes, stream);
+    // float32 gradients (K = V = 64 here; rwkv7_bwd_recurrent takes 128 too): beyond a dozen tokens the chunked
+    // float32 backward, otherwise the token-by-token one
+    if (dtype == RWKV7_DTYPE_F32 && K == 64 && V == 64) {
+        if (T <= RECURRENT_MAX_T)
+            return rwkv7_bwd_recurrent(r, w, k, v, a, b, h0, h0_batch_stride, d_o, d_ht, dr, dw, dk, dv, da, db, dh0,
+                                       B, T, H, K, V, dtype, ws, ws_bytes, stream);
+        int rc = check_seq(r, w, k, v, a, b, h0, h0_batch_stride, dr, nullptr, B, T, H, K, V, dtype, true, true);
+        if (rc != RWKV7_OK) return rc;
+        if (!dw || !dk || !dv || !da || !db) return RWKV7_ERR_NULL_POINTER;
+        if (!aligned16(d_o) || !aligned16(d_ht) || !aligned16(dw) || !aligned16(dk) || !aligned16(dv) ||
+            !aligned16(da) || !aligned16(db) || !aligned16(dh0))
+            return RWKV7_ERR_ALIGNMENT;
+        const size_t need = rwkv7::bwd_chunk_f32_workspace_bytes(B, T, H);
+        if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return RWKV7_ERR_WORKSPACE;
+        rwkv7::BwdArgs p;
+        p.r = r; p.w = w; p.k = k; p.v = v; p.a = a; p.b = b;
+        p.h0 = h0; p.h0_batch_stride = h0 ? h0_batch_stride : 0;
+        p.dO = d_o; p.dht = d_ht;
+        p.dr = dr; p.dw = dw; p.dk = dk; p.dv = dv; p.da = da; p.db = db; p.dh0 = dh0;
+        p.B = B; p.T = T; p.H = H; p.dtype = dtype; p.cu = nullptr;
+        return (int)rwkv7::launch_bwd_chunk_f32(p, ws, static_cast<hipStream_t>(stream));
+    }
     int rc = check_seq(r, w, k, v, a, b, h0, h0_batch_stride, dr, nullptr, B, T, H, K, V, dtype);
     if (rc != RWKV7_OK) return rc;
     if (!dw || !dk || !dv || !da || !db) return RWKV7_ERR_NULL_POINTER;

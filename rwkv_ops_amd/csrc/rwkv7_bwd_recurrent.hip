@@ -75,8 +75,11 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
                           const T* __restrict__ d_o, const float* __restrict__ d_ht,
                           const float* __restrict__ ckpt, float* __restrict__ scratch,
                           T* __restrict__ dr, T* __restrict__ dw, T* __restrict__ dk, T* __restrict__ dv,
-                          T* __restrict__ da, T* __restrict__ db, float* __restrict__ dh0, int T_len, int H)
+                          T* __restrict__ da, T* __restrict__ db, float* __restrict__ dh0, int T_len, int H,
+                          int ckpt_per_head, int ckpt_step, const int* __restrict__ run_if_any, int n_flags)
 {
+    // ckpt: the state before token SEG * s is record ckpt_step * s of this head's ckpt_per_head records.
+    // run_if_any (nullable): n_flags integers; the kernel runs only when one of them is not zero.
     constexpr int CPW = RecShape<N>::CPW, SEG = RecShape<N>::SEG;
     constexpr int VQ = CPW / 4;                  // lanes across a wave's columns, four columns each
     constexpr int ROWS = N / (64 / VQ);          // state rows per lane
@@ -93,6 +96,11 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
     enum { O_DR = 0, O_DK, O_DB, O_DD, O_DA, O_COUNT };
 
     const int tid = threadIdx.x;
+    if (run_if_any != nullptr) {
+        int mine = 0;
+        for (int i = tid; i < n_flags; i += 256) mine |= run_if_any[i];
+        if (__syncthreads_or(mine) == 0) return;
+    }
     const int lane = tid & 63;
     const int wave = tid >> 6;                   // which CPW value columns
     const int bh = blockIdx.x, hi = bh % H;
@@ -103,7 +111,7 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
     const int64_t step = (int64_t)H * N;
     const int64_t base = ((int64_t)(bh / H) * T_len * H + hi) * N;
     const int nseg = (T_len + SEG - 1) / SEG;
-    const float* my_ckpt = ckpt + (int64_t)bh * nseg * (N * N);
+    const float* my_ckpt = ckpt + (int64_t)bh * ckpt_per_head * (N * N);
     float* my_scr = scratch + (int64_t)bh * SEG * (N * N);
 
     // one block of per-token vectors -> LDS as float (w as the decay d, and as dfac = dd/dw = -exp(w) d)
@@ -166,7 +174,7 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
         // ---- the segment forward once more: the state before each token -> scratch, sa -> LDS
         {
             float4_t s[ROWS];
-            const float* src = my_ckpt + (int64_t)seg * (N * N) + tile;
+            const float* src = my_ckpt + (int64_t)seg * ckpt_step * (N * N) + tile;
 #pragma unroll
             for (int i = 0; i < ROWS; ++i) s[i] = *reinterpret_cast<const float4_t*>(src + i * N);
             for (int t0 = 0; t0 < slen; t0 += RB_TB) {
@@ -278,7 +286,9 @@ template <int N> constexpr size_t rec_lds_bytes() {
 }
 
 template <typename T, int N>
-hipError_t launch_bwd_rec_t(const BwdArgs& p, const float* ckpt, float* scratch, hipStream_t stream) {
+hipError_t launch_bwd_rec_t(const BwdArgs& p, const float* ckpt, float* scratch, hipStream_t stream,
+                            int ckpt_per_head = 0, int ckpt_step = 1, const int* run_if_any = nullptr, int n_flags = 0) {
+    if (ckpt_per_head == 0) ckpt_per_head = (p.T + RecShape<N>::SEG - 1) / RecShape<N>::SEG;
     constexpr size_t lds = rec_lds_bytes<N>();
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_recurrent_kernel<T, N>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -286,10 +296,17 @@ hipError_t launch_bwd_rec_t(const BwdArgs& p, const float* ckpt, float* scratch,
     bwd_recurrent_kernel<T, N><<<dim3((unsigned)(p.B * p.H)), dim3(256), lds, stream>>>(
         (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, (const T*)p.a, (const T*)p.b,
         (const T*)p.dO, p.dht, ckpt, scratch, (T*)p.dr, (T*)p.dw, (T*)p.dk, (T*)p.dv, (T*)p.da, (T*)p.db,
-        p.dh0, p.T, p.H);
+        p.dh0, p.T, p.H, ckpt_per_head, ckpt_step, run_if_any, n_flags);
     return hipGetLastError();
 }
 }  // namespace
+
+// the walk alone, for float32 tensors at K = V = 64, over states stored every 16 tokens (record 4 s = the state
+// before token 64 s); it runs only when one of the n_flags integers at run_if_any is not zero
+hipError_t launch_bwd_recurrent_walk_f32(const BwdArgs& p, const float* states16, float* scratch,
+                                         const int* run_if_any, int n_flags, hipStream_t stream) {
+    return launch_bwd_rec_t<float, 64>(p, states16, scratch, stream, (p.T + 15) / 16, 4, run_if_any, n_flags);
+}
 
 hipError_t launch_bwd_recurrent(const BwdArgs& p, int N, void* ws, hipStream_t stream) {
     const int seg = bwd_recurrent_segment(N);

@@ -1,0 +1,36 @@
+// What the float32 chunk kernels (16-token chunks on the float32 matrix cores, K = V = 64) share: the register
+// layouts are described at the top of rwkv7_fwd_chunk_f32.hip.
+#pragma once
+#include "rwkv7_chunk.h"
+
+namespace rwkv7 {
+
+constexpr int C16 = 16;                        // tokens per chunk
+constexpr int NH = 64;                         // head size
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float G_MIN2 = G_MIN * LOG2E;        // per-step log-decay clamp, in base-2 units
+// A chunk whose total log decay exceeds this (in some channel) is walked token by token: k e^{-gi} must stay
+// well inside float32 (e^60 times |k|); RWKV7's own decay range gives at most 16 * 0.607 = 9.7.
+constexpr float STRONG2 = 60.f * LOG2E;
+__device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+constexpr int LDF = 68;                        // row stride (floats) of the row-major tiles [16 tokens][64 channels]
+constexpr int TILE_F = C16 * LDF * 4;          // bytes of a row-major tile
+
+__device__ __forceinline__ float4_t mfma_f32(float a, float b, float4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+}
+// sum over the 16 lanes of a DPP row, delivered to all of them
+__device__ __forceinline__ float row_sum(float x) {
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x121, 0xf, 0xf, true));   // row_ror:1
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x122, 0xf, 0xf, true));   // row_ror:2
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x124, 0xf, 0xf, true));   // row_ror:4
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x128, 0xf, 0xf, true));   // row_ror:8
+    return x;
+}
+// row `row`, columns col .. col + 3 of a tile
+__device__ __forceinline__ float4_t tile4(const unsigned char* smem, int off, int row, int col) {
+    return *reinterpret_cast<const float4_t*>(smem + off + (row * LDF + col) * 4);
+}
+
+}  // namespace rwkv7

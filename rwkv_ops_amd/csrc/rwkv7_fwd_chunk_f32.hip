@@ -24,7 +24,7 @@
 // are all the inverse needs:  R(Z1 Z2) = mfma(A = R(Z1^T), B = R(Z2)).
 // Operands that come from the inputs lie in LDS as row-major float32 tiles [token][channel]; "row x, four
 // consecutive columns" is one 16-byte read and serves four instructions.
-#include "rwkv7_chunk.h"
+#include "rwkv7_f32_mma.h"
 #include "rwkv7_kernels.h"
 #include "../../include/rwkv7_mi355x.h"
 
@@ -32,18 +32,7 @@ namespace rwkv7 {
 
 namespace {
 
-constexpr int C16 = 16;                        // tokens per chunk
-constexpr int NH = 64;                         // head size
-constexpr float LOG2E = 1.4426950408889634f;
-constexpr float G_MIN2 = G_MIN * LOG2E;        // per-step log-decay clamp, in base-2 units
-// A chunk whose total log decay exceeds this (in some channel) is walked token by token: k e^{-gi} must stay
-// well inside float32 (e^60 times |k|); RWKV7's own decay range gives at most 16 * 0.607 = 9.7.
-constexpr float STRONG2 = 60.f * LOG2E;
-__device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-constexpr int LDF = 68;                        // row stride (floats) of the row-major tiles [16 tokens][64 channels]
 constexpr int LDC = 20;                        // row stride (floats) of the transposed tiles [64 channels][16 tokens]
-constexpr int TILE_F = C16 * LDF * 4;          // bytes of a row-major tile
 constexpr int TILE_C = NH * LDC * 4;           // bytes of a transposed one (large enough to hold a row-major tile too)
 static_assert(TILE_C >= TILE_F, "the strong-decay path keeps a row-major tile in a transposed tile's place");
 // one buffer = everything the consumer waves need of one chunk; three buffers, chunk c in buffer c % 3
@@ -57,22 +46,6 @@ constexpr int BUF_BYTES = F_SCR + 1024;
 constexpr int F_DEC = F_QG, F_RAW_R = F_KGT;   // strong chunks: per-step decays and raw r (row-major) in these places
 constexpr int LDS_F32_BYTES = 3 * BUF_BYTES;
 static_assert(LDS_F32_BYTES <= 160 * 1024, "one workgroup per CU");
-
-__device__ __forceinline__ float4_t mfma_f32(float a, float b, float4_t c) {
-    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
-}
-// sum over the 16 lanes of a DPP row, delivered to all of them
-__device__ __forceinline__ float row_sum(float x) {
-    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x121, 0xf, 0xf, true));   // row_ror:1
-    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x122, 0xf, 0xf, true));   // row_ror:2
-    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x124, 0xf, 0xf, true));   // row_ror:4
-    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x128, 0xf, 0xf, true));   // row_ror:8
-    return x;
-}
-// row `row`, columns col .. col + 3 of a tile
-__device__ __forceinline__ float4_t tile4(const unsigned char* smem, int off, int row, int col) {
-    return *reinterpret_cast<const float4_t*>(smem + off + (row * LDF + col) * 4);
-}
 
 }  // namespace
 
@@ -88,10 +61,11 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
                             const float* __restrict__ v_, const float* __restrict__ a_, const float* __restrict__ b_,
                             const float* __restrict__ h0, int64_t h0_batch_stride, const int* __restrict__ h0_map,
                             int n_state, float* __restrict__ o_, float* __restrict__ ht, SeqLayout L,
-                            float* __restrict__ seg_states, int seg)
+                            float* __restrict__ seg_states, int seg, int* __restrict__ strong_out)
 {
     // seg_states (dense batches): the state BEFORE token t is stored for every t that is a multiple of `seg` (a
-    // multiple of 16), [workgroup][t / seg][64][64]: what the recurrent backward restarts from.  o_ may then be NULL.
+    // multiple of 16), [workgroup][t / seg][64][64]: what the backward kernels restart from.  o_ may then be NULL.
+    // strong_out (nullable): one integer per workgroup, 1 when a chunk of its sequence was walked token by token.
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_all[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int w = wave & 3;                    // consumers: value columns 16 w .. + 15; producers: channels 16 w .. + 15
@@ -102,6 +76,7 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
     const int T = sp.len, NT = (T + C16 - 1) / C16;
     const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
     if (NT == 0) {                             // a sequence without tokens: the state passes through
+        if (strong_out != nullptr && threadIdx.x == 0) strong_out[bh] = 0;
         if (!producer && ht != nullptr) {
             const int x = threadIdx.x & 15, g = (threadIdx.x & 63) >> 4;
             float* dst = ht + (int64_t)bh * (NH * NH) + 16 * w + x;
@@ -277,6 +252,7 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
     }
     __syncthreads();                           // rounds 0 and 1: the first chunk is on its way
     __syncthreads();
+    bool any_strong = false;
     for (int c = 0; c < NT; ++c) {             // round c + 2
         int lane = threadIdx.x & 63;
         asm volatile("" : "+v"(lane));
@@ -295,6 +271,7 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
             const int* fl = reinterpret_cast<const int*>(smem + F_FLAG);
             strong = (fl[0] | fl[1] | fl[2] | fl[3]) != 0;
         }
+        any_strong |= strong;
         if (strong) {
             // token by token in float32 on the state as it lies in the registers
             const int nt = T - c * C16 < C16 ? T - c * C16 : C16;
@@ -378,6 +355,7 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
             *reinterpret_cast<float4_t*>(o_ + ((sp.tok0 + c * C16 + x) * H + hi) * NH + 16 * w + 4 * g) = OT;
         __syncthreads();
     }
+    if (strong_out != nullptr && threadIdx.x == 0) strong_out[bh] = any_strong ? 1 : 0;
     if (ht != nullptr) {
         const int x = threadIdx.x & 15, g = (threadIdx.x & 63) >> 4;
         float* dst = ht + (int64_t)bh * (NH * NH) + 16 * w + x;
@@ -399,19 +377,21 @@ hipError_t launch_fwd_chunk_f32(const SeqArgs& p, hipStream_t stream) {
     chunk16_f32_fwd_kernel<<<dim3((unsigned)(p.B * p.H)), dim3(768), LDS_F32_BYTES, stream>>>(
         (const float*)p.r, (const float*)p.w, (const float*)p.k, (const float*)p.v, (const float*)p.a,
         (const float*)p.b, p.h0, p.h0_batch_stride, p.h0_map, p.n_state, (float*)p.o, p.ht, seq_layout(p, nullptr),
-        nullptr, 0);
+        nullptr, 0, nullptr);
     return hipGetLastError();
 }
 
 // the forward without outputs, storing the state at the start of every segment of `seg` tokens (dense batches,
-// float32 tensors, K = V = 64; seg a multiple of 16)
-hipError_t launch_fwd_chunk_f32_states(const SeqArgs& p, float* states, int seg, hipStream_t stream) {
+// float32 tensors, K = V = 64; seg a multiple of 16); strong (nullable): per (batch, head) whether a chunk's decay was
+// too strong for the chunk form
+hipError_t launch_fwd_chunk_f32_states(const SeqArgs& p, float* states, int seg, hipStream_t stream, int* strong) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(chunk16_f32_fwd_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, LDS_F32_BYTES);
     if (e != hipSuccess) return e;
     chunk16_f32_fwd_kernel<<<dim3((unsigned)(p.B * p.H)), dim3(768), LDS_F32_BYTES, stream>>>(
         (const float*)p.r, (const float*)p.w, (const float*)p.k, (const float*)p.v, (const float*)p.a,
-        (const float*)p.b, p.h0, p.h0_batch_stride, nullptr, 0, nullptr, nullptr, seq_layout(p, nullptr), states, seg);
+        (const float*)p.b, p.h0, p.h0_batch_stride, nullptr, 0, nullptr, nullptr, seq_layout(p, nullptr), states, seg,
+        strong);
     return hipGetLastError();
 }
 

@@ -153,7 +153,7 @@ def rwkv7_bwd(r: torch.Tensor, w: torch.Tensor, k: torch.Tensor, v: torch.Tensor
               d_o: Optional[torch.Tensor], d_ht: Optional[torch.Tensor]
               ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
                          torch.Tensor, torch.Tensor]:
-    """Gradients of ``rwkv7_fwd``: bf16 ``[B, T, H, 64]`` inputs (contiguous), ``d_o`` like ``r`` or
+    """Gradients of ``rwkv7_fwd``: bf16 or float32 ``[B, T, H, 64]`` inputs (contiguous), ``d_o`` like ``r`` or
     None, ``d_ht`` float32 ``[B, H, 64, 64]`` or None.  Returns ``(dr, dw, dk, dv, da, db, dh0)`` with
     ``dh0`` float32 ``[B, H, 64, 64]`` (per batch entry, also when ``h0`` is a broadcast ``[1, ...]``)."""
     lib = _lib.load()
@@ -221,9 +221,13 @@ def _fwd_backward(ctx, d_o, d_ht):
     d_ht_c = None
     if ctx.want_state and d_ht is not None and d_ht.numel() > 0:
         d_ht_c = d_ht.to(torch.float32).contiguous()
-    if dt == torch.float32 or r.shape[-1] != HEAD_SIZE:
-        # float32 calls get float32 gradients, and head size 128 has no chunked backward: both take the
-        # float32 recurrent backward, which reads any of the three dtypes as it is
+    if dt == torch.float32 and r.shape[-1] == HEAD_SIZE:
+        # float32 calls get float32 gradients: the chunked float32 backward (a dozen tokens or fewer: the recurrent one)
+        d_o_c = None if d_o is None else d_o.to(dt).contiguous()
+        dr, dw, dk, dv, da, db, dh0 = torch.ops.rwkv_ops_amd.rwkv7_bwd(r, w, k, v, a, b, h0, d_o_c, d_ht_c)
+    elif r.shape[-1] != HEAD_SIZE:
+        # head size 128 has no chunked backward: the float32 recurrent backward, which reads any of the three
+        # dtypes as it is
         d_o_c = None if d_o is None else d_o.to(dt).contiguous()
         dr, dw, dk, dv, da, db, dh0 = torch.ops.rwkv_ops_amd.rwkv7_bwd_recurrent(
             r, w, k, v, a, b, h0, d_o_c, d_ht_c)

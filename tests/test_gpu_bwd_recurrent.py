@@ -89,18 +89,22 @@ def test_recurrent_backward_variants(device):
                 assert float(a_[:, T - pad:].abs().max()) == 0.0, n
 
 
-def test_rwkv7_bwd_routes_float32_to_the_recurrent_backward(device):
+def test_rwkv7_bwd_routes_short_float32_calls_to_the_recurrent_backward(device):
+    """A dozen tokens or fewer: rwkv7_bwd on float32 tensors is the recurrent backward, bit for bit; longer calls
+    take the chunked float32 backward (tests/test_gpu_bwd_chunk_f32.py), a different order of the same arithmetic."""
     lib = _lib.load()
-    B, T, H, N = 1, 100, 2, 64
-    xs = make_inputs(B, T, H, N, seed=3200, dtype=torch.float32)
-    g = torch.Generator().manual_seed(4)
-    dO = torch.randn(B, T, H, N, generator=g)
-    dS = 0.1 * torch.randn(B, H, N, N, generator=g)
-    a_ = run(lib, device, xs, dO, dS, N, torch.float32, entry="rwkv7_bwd")
-    b_ = run(lib, device, xs, dO, dS, N, torch.float32)
-    for x, y in zip(a_, b_):
-        assert torch.equal(x, y)
-    assert lib.rwkv7_bwd_workspace_bytes(B, T, H, _lib.DTYPE_F32) == lib.rwkv7_bwd_recurrent_workspace_bytes(B, T, H, 64)
+    N = 64
+    for B, T, H, same in ((1, 12, 2, True), (2, 5, 1, True), (1, 100, 2, False)):
+        xs = make_inputs(B, T, H, N, seed=3200, dtype=torch.float32)
+        g = torch.Generator().manual_seed(4)
+        dO = torch.randn(B, T, H, N, generator=g)
+        dS = 0.1 * torch.randn(B, H, N, N, generator=g)
+        a_ = run(lib, device, xs, dO, dS, N, torch.float32, entry="rwkv7_bwd")
+        b_ = run(lib, device, xs, dO, dS, N, torch.float32)
+        for x, y in zip(a_, b_):
+            assert torch.equal(x, y) if same else rel_l2(x, y) < 1e-5
+        if same:
+            assert lib.rwkv7_bwd_workspace_bytes(B, T, H, _lib.DTYPE_F32) == lib.rwkv7_bwd_recurrent_workspace_bytes(B, T, H, 64)
 
 
 def test_recurrent_and_chunked_backward_agree(device):
