@@ -23,7 +23,8 @@
 //   2. chunk16_f32_bwd_grad_kernel, one workgroup per (batch, head, chunk), no chain: the dA matrices and the six
 //      gradients that are [token][key channel];
 // A chunk whose decay is too strong for k e^{-gi} (never with RWKV7's own parameterisation) has no chunk form
-// here: the forward pass leaves a flag per (batch, head), and when any is set both kernels return at once and
+// here: the forward pass leaves a flag per (batch, head), and when any is set the first kernel returns at once,
+// the second stores nothing, and
 //   3. the token-by-token kernel of rwkv7_bwd_recurrent.hip, which otherwise returns at once, does the whole call.
 #include "rwkv7_f32_mma.h"
 #include "rwkv7_kernels.h"
@@ -362,7 +363,9 @@ constexpr int LDX = 20;                        // row stride (floats) of a wave'
 constexpr int G_TR = G_BOX + 8 * 1024;         // per wave four areas [16 tokens][LDX]
 constexpr int TR_BYTES = 16 * LDX * 4;
 constexpr int G_HD = G_TR + 4 * 4 * TR_BYTES;  // per wave float [16]
-constexpr int LDS_GRAD_BYTES = G_HD + 4 * 64;
+constexpr int G_V = G_HD + 4 * 64, G_DO = G_V + TILE_F, G_SA = G_DO + TILE_F, G_DY = G_SA + TILE_F;   // row-major tiles
+constexpr int G_OUT5 = G_DY + TILE_F;           // a fifth tile: the results leave through the four above and this one
+constexpr int LDS_GRAD_BYTES = G_OUT5 + TILE_F;
 }  // namespace
 
 // One workgroup of four waves per (batch, head, chunk); wave w owns key channels 16 w .. + 15, lane (x, g) token x
@@ -378,7 +381,9 @@ void chunk16_f32_bwd_grad_kernel(const float* __restrict__ r_, const float* __re
                                  float* __restrict__ da_, float* __restrict__ db_, int B, int T, int H)
 {
     __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_GRAD_BYTES];
-    if (any_strong(strong_flags, B * H)) return;
+    // (the forward pass's flags are asked for now and looked at only before the stores: nothing here waits for them)
+    int flagged = 0;
+    for (int i = threadIdx.x; i < B * H; i += 256) flagged |= strong_flags[i];
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int x = lane & 15, g = lane >> 4;
@@ -390,62 +395,30 @@ void chunk16_f32_bwd_grad_kernel(const float* __restrict__ r_, const float* __re
     const int64_t row = (((int64_t)bi * T + (valid ? t : T - 1)) * H + hi) * NH;
     const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 
-    // ---- loads.  Full rows [token x][16 vt + 4 g .. + 3] of V, dO, SA, dY: both operands of the dA products and
-    // the B operands of the products with h and dh
-    float4_t V4[4], D4[4], S4[4], Y4[4];
-#pragma unroll
-    for (int vt = 0; vt < 4; ++vt) {
-        V4[vt] = *reinterpret_cast<const float4_t*>(v_ + row + 16 * vt + 4 * g);
-        D4[vt] = do_ != nullptr ? *reinterpret_cast<const float4_t*>(do_ + row + 16 * vt + 4 * g) : zero4;
-        S4[vt] = *reinterpret_cast<const float4_t*>(sa_ws + rec * (C16 * NH) + x * NH + 16 * vt + 4 * g);
-        Y4[vt] = *reinterpret_cast<const float4_t*>(dy_ws + rec * (C16 * NH) + x * NH + 16 * vt + 4 * g);
-    }
+    // ---- this wave's channels of the inputs, scaled, and four of the scaled operands transposed:
+    // T(X)[e] = X[token 4 g + e][channel 16 w + x]
     const int ch = 16 * w + 4 * g;
     float4_t W4 = *reinterpret_cast<const float4_t*>(w_ + row + ch), R4 = *reinterpret_cast<const float4_t*>(r_ + row + ch);
     float4_t K4 = *reinterpret_cast<const float4_t*>(k_ + row + ch), A4 = *reinterpret_cast<const float4_t*>(a_ + row + ch);
     float4_t B4 = *reinterpret_cast<const float4_t*>(b_ + row + ch);
-    // h and dh as A operands: row (key channel) 16 w + x, values 16 vt + 4 g .. + 3
-    float4_t hA[4], dhA[4];
-#pragma unroll
-    for (int vt = 0; vt < 4; ++vt) {
-        hA[vt] = *reinterpret_cast<const float4_t*>(states + rec * (NH * NH) + (16 * w + x) * NH + 16 * vt + 4 * g);
-        dhA[vt] = *reinterpret_cast<const float4_t*>(dhs + rec * (NH * NH) + (16 * w + x) * NH + 16 * vt + 4 * g);
-    }
-    if (!valid) {
-        R4 = K4 = A4 = B4 = zero4;
-#pragma unroll
-        for (int vt = 0; vt < 4; ++vt) V4[vt] = D4[vt] = zero4;
-    }
-
-    // ---- the dA matrix of this wave, as R(dA^T) (row i = x, column j = 4 g + e) and as R(dA)
-    {
-        // gram(X, Y): lane (x, g) gets sum_v X[4 g + e][v] Y[x][v]
-        auto gram = [&](const float4_t (&X)[4], const float4_t (&Y)[4]) {
-            float4_t acc = zero4;
-#pragma unroll
-            for (int vt = 0; vt < 4; ++vt)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) acc = mfma_f32(X[vt][e], Y[vt][e], acc);
-            return acc;
-        };
-        const bool strict = w >= 2;                                  // dAak, dAab keep j < i
-        float4_t f1, f2;                                             // dA[i][j] = left_i . right_j
-        if (w == 0)      { f1 = gram(V4, D4); f2 = gram(D4, V4); }   // dAqk = dO V^T
-        else if (w == 1) { f1 = gram(S4, D4); f2 = gram(D4, S4); }   // dAqb = dO SA^T
-        else if (w == 2) { f1 = gram(V4, Y4); f2 = gram(Y4, V4); }   // dAak = dY V^T
-        else             { f1 = gram(S4, Y4); f2 = gram(Y4, S4); }   // dAab = dY SA^T
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int j1 = 4 * g + e, i1 = x;                        // f1: dA[i = x][j = 4 g + e]
-            const int i2 = 4 * g + e, j2 = x;                        // f2: dA[i = 4 g + e][j = x]
-            if (strict ? j1 >= i1 : j1 > i1) f1[e] = 0.f;
-            if (strict ? j2 >= i2 : j2 > i2) f2[e] = 0.f;
-        }
-        *reinterpret_cast<float4_t*>(smem + G_BOX + (2 * w) * 1024 + lane * 16) = f1;
-        *reinterpret_cast<float4_t*>(smem + G_BOX + (2 * w + 1) * 1024 + lane * 16) = f2;
-    }
-
-    // ---- this wave's channels of the scaled operands, and four of them transposed: T(X)[e] = X[token 4 g + e][channel 16 w + x]
+    // V, dO, SA, dY of the chunk ([token][value], all of which every wave needs: both operands of the dA products and
+    // the B operands of the products with h and dh): each wave fetches its sixteen columns, through LDS to all
+    float4_t Vq = *reinterpret_cast<const float4_t*>(v_ + row + ch);
+    float4_t Dq = do_ != nullptr ? *reinterpret_cast<const float4_t*>(do_ + row + ch) : zero4;
+    const float4_t Sq = *reinterpret_cast<const float4_t*>(sa_ws + rec * (C16 * NH) + x * NH + ch);
+    const float4_t Yq = *reinterpret_cast<const float4_t*>(dy_ws + rec * (C16 * NH) + x * NH + ch);
+    // One slab = thirty-two value columns of h and dh, rows [key channel 16 w + x][16 vt + 4 g .. + 3] for two vt
+    // (their A operands): the two 64-byte halves of every 128-byte line are requested back to back, so that the second
+    // request finds the first one's miss in flight.  The next slab is on its way while this one is multiplied.
+    struct Slab { float4_t h[2], dh[2]; };
+    auto load_slab = [&](Slab& sl, int pair) {
+        const int64_t at = rec * (NH * NH) + (16 * w + x) * NH + 32 * pair + 4 * g;
+        sl.h[0] = *reinterpret_cast<const float4_t*>(states + at); sl.h[1] = *reinterpret_cast<const float4_t*>(states + at + 16);
+        sl.dh[0] = *reinterpret_cast<const float4_t*>(dhs + at);   sl.dh[1] = *reinterpret_cast<const float4_t*>(dhs + at + 16);
+    };
+    Slab nxt;
+    load_slab(nxt, 0);
+    if (!valid) R4 = K4 = A4 = B4 = zero4;
     Scaled s;
     scale_inputs(s, valid, W4, R4, K4, A4, B4);
     float4_t Tqg, Tag, Tkt, Tbt;
@@ -463,32 +436,63 @@ void chunk16_f32_bwd_grad_kernel(const float* __restrict__ r_, const float* __re
             Tbt[e] = tr[3 * 16 * LDX + (4 * g + e) * LDX + x];
         }
     }
+
+    // ---- the products over the value columns.  The dA matrix of this wave, dA[i][j] = left_i . right_j
+    // (0: dAqk = dO V^T, 1: dAqb = dO SA^T, 2: dAak = dY V^T, 3: dAab = dY SA^T), as f1 = R(dA^T) (row i = x, column
+    // j = 4 g + e) and f2 = R(dA); and the four products that need no dA, R(dX^T)[channel 4 g + e][token x].
+    float4_t f1 = zero4, f2 = zero4, dqg = zero4, dag = zero4, dkg = zero4, dbg = zero4, hdp = zero4;
+    {
+        if (!valid) Vq = Dq = zero4;               // rows past the end
+        auto put4 = [&](int off, float4_t val) { *reinterpret_cast<float4_t*>(smem + off + (x * LDF + ch) * 4) = val; };
+        put4(G_V, Vq); put4(G_DO, Dq); put4(G_SA, Sq); put4(G_DY, Yq);
+    }
+    __syncthreads();
+#pragma unroll 1
+    for (int pair = 0; pair < 2; ++pair) {
+        Slab cur = nxt;
+        load_slab(nxt, 1);
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int col = 32 * pair + 16 * half + 4 * g;
+            const float4_t V4 = tile4(smem, G_V, x, col), D4 = tile4(smem, G_DO, x, col);
+            const float4_t S4 = tile4(smem, G_SA, x, col), Y4 = tile4(smem, G_DY, x, col);
+            const float4_t right = (w & 1) ? S4 : V4, left = (w & 2) ? Y4 : D4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                // gram(X, Y): lane (x, g) gets sum_v X[4 g + e][v] Y[x][v]
+                f1 = mfma_f32(right[e], left[e], f1);
+                f2 = mfma_f32(left[e], right[e], f2);
+                dqg = mfma_f32(cur.h[half][e], D4[e], dqg);              // h dO^T
+                dkg = mfma_f32(cur.dh[half][e], V4[e], dkg);             // dh V^T
+                dag = mfma_f32(cur.h[half][e], Y4[e], dag);              // h dY^T
+                dbg = mfma_f32(cur.dh[half][e], S4[e], dbg);             // dh SA^T
+            }
+            hdp += cur.h[half] * cur.dh[half];
+        }
+    }
+    {
+        const bool strict = w >= 2;                                  // dAak, dAab keep j < i
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int j1 = 4 * g + e, i1 = x;                        // f1: dA[i = x][j = 4 g + e]
+            const int i2 = 4 * g + e, j2 = x;                        // f2: dA[i = 4 g + e][j = x]
+            if (strict ? j1 >= i1 : j1 > i1) f1[e] = 0.f;
+            if (strict ? j2 >= i2 : j2 > i2) f2[e] = 0.f;
+        }
+        *reinterpret_cast<float4_t*>(smem + G_BOX + (2 * w) * 1024 + lane * 16) = f1;
+        *reinterpret_cast<float4_t*>(smem + G_BOX + (2 * w + 1) * 1024 + lane * 16) = f2;
+    }
     // rowsum(h * dh) of channel 16 w + x, brought to the lanes that own the channel
     float4_t hd4;
     {
-        float4_t p = zero4;
-#pragma unroll
-        for (int vt = 0; vt < 4; ++vt) p += hA[vt] * dhA[vt];
-        float hd = (p[0] + p[1]) + (p[2] + p[3]);
+        float hd = (hdp[0] + hdp[1]) + (hdp[2] + hdp[3]);
         hd += __shfl_xor(hd, 16, 64);
         hd += __shfl_xor(hd, 32, 64);
         float* hdl = reinterpret_cast<float*>(smem + G_HD + w * 64);
         if (g == 0) hdl[x] = hd;
         hd4 = *reinterpret_cast<const float4_t*>(hdl + 4 * g);
     }
-
-    // ---- the products that need no dA: R(dX^T)[channel 4 g + e][token x]
-    float4_t dqg = zero4, dag = zero4, dkg = zero4, dbg = zero4;
-#pragma unroll
-    for (int vt = 0; vt < 4; ++vt)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            dqg = mfma_f32(hA[vt][e], D4[vt][e], dqg);               // h dO^T
-            dkg = mfma_f32(dhA[vt][e], V4[vt][e], dkg);              // dh V^T
-            dag = mfma_f32(hA[vt][e], Y4[vt][e], dag);               // h dY^T
-            dbg = mfma_f32(dhA[vt][e], S4[vt][e], dbg);              // dh SA^T
-        }
-    __syncthreads();
+    const bool strong = __syncthreads_or(flagged) != 0;     // then the token-by-token kernel does the whole call
     auto box = [&](int i) { return *reinterpret_cast<const float4_t*>(smem + G_BOX + i * 1024 + lane * 16); };
     float4_t dkt = zero4, dbt = zero4;
     {
@@ -530,11 +534,24 @@ void chunk16_f32_bwd_grad_kernel(const float* __restrict__ r_, const float* __re
         const float gnat = s.gstep[e] > G_MIN2 ? s.gstep[e] * (1.f / LOG2E) : 0.f;
         dw[e] = (after_gi + after_ge + dG) * gnat;
     }
-    if (valid) {
-        const int64_t o = (((int64_t)bi * T + t) * H + hi) * NH + ch;
-        *reinterpret_cast<float4_t*>(dr_ + o) = dr; *reinterpret_cast<float4_t*>(dw_ + o) = dw;
-        *reinterpret_cast<float4_t*>(dk_ + o) = dk; *reinterpret_cast<float4_t*>(da_ + o) = da;
-        *reinterpret_cast<float4_t*>(db_ + o) = db;
+    // The results go through LDS so that a wave stores whole 256-byte rows (tokens 4 w .. + 3, lane = sixteen bytes
+    // of a row) instead of a 64-byte piece of each of sixteen rows.  (The four tiles of the inputs have been read by
+    // everybody before the last barrier.)
+    {
+        auto put4 = [&](int off, float4_t val) { *reinterpret_cast<float4_t*>(smem + off + (x * LDF + ch) * 4) = val; };
+        put4(G_V, dr); put4(G_DO, dw); put4(G_SA, dk); put4(G_DY, da); put4(G_OUT5, db);
+    }
+    __syncthreads();
+    {
+        const int tok = 4 * w + g, piece = 4 * x, ts = c * C16 + tok;
+        if (ts < T && !strong) {
+            const int64_t o = (((int64_t)bi * T + ts) * H + hi) * NH + piece;
+            *reinterpret_cast<float4_t*>(dr_ + o) = tile4(smem, G_V, tok, piece);
+            *reinterpret_cast<float4_t*>(dw_ + o) = tile4(smem, G_DO, tok, piece);
+            *reinterpret_cast<float4_t*>(dk_ + o) = tile4(smem, G_SA, tok, piece);
+            *reinterpret_cast<float4_t*>(da_ + o) = tile4(smem, G_DY, tok, piece);
+            *reinterpret_cast<float4_t*>(db_ + o) = tile4(smem, G_OUT5, tok, piece);
+        }
     }
 }
 
