@@ -339,7 +339,9 @@ def main():
     f32_bytes = 7 * B * T * H * N * 4 + 2 * B * H * N * N * 4
     del x32, o32
 
-    # float32 gradients at the training shape: the float32 recurrent backward (rwkv7_bwd with float32 tensors)
+    # float32 gradients at the training shape: the chunked float32 backward on the float32 matrix cores (rwkv7_bwd
+    # with float32 tensors: the state before every 16-token chunk from one more forward pass, a chain kernel and a
+    # per-chunk gradient kernel)
     xb32 = [t.float() for t in xb[:6]]
     d_o32 = d_o.float()
     g32 = [torch.empty_like(xb32[0]) for _ in range(6)]
@@ -351,7 +353,10 @@ def main():
                            *[ptr(g) for g in g32], ptr(dh0), Bb, Tb, Hb, N, N, 1, ptr(rws), rws_bytes, stream)
         assert rc == 0, rc
 
-    ms_bwd_f32, _ = time_gpu(bwd_f32, max(3, args.steps // 40), 1, torch)
+    ms_bwd_f32, _ = time_gpu(bwd_f32, max(5, args.steps // 10), 2, torch)
+    # what the three kernels move per 16-token chunk and head: the forward pass 24 KiB in + 16 KiB state out, the
+    # chain kernel 28 + 16 in and 16 (dh) + 8 (SA, dY) + 4 (dv) out, the gradient kernel 88 in and out
+    bwd_f32_traffic = Bb * Hb * ((Tb + 15) // 16) * 200 * 1024
     del xb32, d_o32, g32, rws
 
     # ------------------------------------------------------------------ head size 128 (bf16, chunked forward)
@@ -492,9 +497,11 @@ def main():
                     # consumer waves, 96 by the producers, 2048 flops each (v_mfma_f32_16x16x4_f32)
                     "mfma_f32_executed_tflops": (B * H * ((T + 15) // 16) * 416 * 2048) / (ms_f32 * 1e-3) / 1e12,
                     "mfma_f32_frac_of_peak": (B * H * ((T + 15) // 16) * 416 * 2048) / (ms_f32 * 1e-3) / 157.3e12},
-        "float32_backward": {"workload": f"rwkv7_bwd on float32 tensors (the float32 recurrent backward, forward states "
-                                         f"recomputed inside), B={Bb} T={Tb} H={Hb}, all seven gradients",
-                             "ms": ms_bwd_f32, "us_per_token": ms_bwd_f32 * 1e3 / Tb},
+        "float32_backward": {"workload": f"rwkv7_bwd on float32 tensors (the chunked float32 backward on the float32 matrix "
+                                         f"cores, forward states recomputed inside), B={Bb} T={Tb} H={Hb}, all seven gradients",
+                             "ms": ms_bwd_f32, "us_per_token": ms_bwd_f32 * 1e3 / Tb,
+                             "kernel_traffic_bytes": bwd_f32_traffic,
+                             "kernel_traffic_frac_of_hbm_peak": bwd_f32_traffic / (ms_bwd_f32 * 1e-3) / HBM_PEAK},
         "head128": {"workload": f"rwkv7_fwd, K=V=128, B={B2} T={T2} H={H2} bf16 (the chunked kernel for that head size: one "
                                 "workgroup per (batch, head), state in registers), float32 states in and out",
                     "ms": ms_128, "tokens_per_s": B2 * T2 / (ms_128 * 1e-3), "us_per_chunk": ms_128 * 1e3 / (T2 // 64),

@@ -202,9 +202,15 @@ int rwkv7_fwd_chunk_scan(const float* h0, int64_t h0_batch_stride, void* o, floa
  * the gradient with respect to the API's `w` argument) and, if dh0 != NULL, the
  * gradient of the initial state (float32 [B,H,64,64], one per batch entry even when
  * h0 is broadcast).  Forward intermediates are recomputed, nothing is saved by the
- * forward call.  bf16 runs the chunked MFMA backward; f32 (K = V = 64) runs
- * rwkv7_bwd_recurrent below and needs its, larger, workspace
- * (rwkv7_bwd_workspace_bytes answers for the dtype it is asked about). */
+ * forward call.  bf16 runs the chunked MFMA backward; f32 (K = V = 64) beyond 12 tokens
+ * runs the chunked float32 backward (16-token chunks on the float32 matrix cores: one more
+ * forward pass that stores the state before every chunk, a kernel that walks the chain of
+ * adjoint states per (batch, head), a kernel per (batch, head, chunk) for the rest; a call
+ * in which some chunk's total decay is below e^-60 is done token by token instead, by the
+ * kernel of rwkv7_bwd_recurrent, inside the same call), at most 12 tokens
+ * rwkv7_bwd_recurrent below.  The float32 workspace is the larger one: 40 KiB per 16 tokens
+ * and head plus 1 MiB per head (rwkv7_bwd_workspace_bytes answers for the dtype it is asked
+ * about). */
 size_t rwkv7_bwd_workspace_bytes(int B, int T, int H, int dtype);
 int rwkv7_bwd(const void* r, const void* w, const void* k, const void* v,
               const void* a, const void* b,
@@ -217,8 +223,8 @@ int rwkv7_bwd(const void* r, const void* w, const void* k, const void* v,
 /* The backward of the reference's native loop (native_keras_op.py:80-88, differentiated there by the host
  * framework's autograd) one token at a time in float32 arithmetic, for either dtype of the tensors
  * (bf16, f32, f16: values are widened on load, gradients rounded on store) and K = V = 64 or 128: the
- * accurate path -- float32 callers, head size 128, float16 -- several microseconds per token, not the
- * throughput path.  Same arguments and meaning as rwkv7_bwd; dense batches only.  The workspace
+ * token-by-token path -- head size 128, float16, float32 calls of a dozen tokens or with very strong decays --
+ * several microseconds per token, not the throughput path.  Same arguments and meaning as rwkv7_bwd; dense batches only.  The workspace
  * (rwkv7_bwd_recurrent_workspace_bytes: the state of every (batch, head) at the start of each 64-token
  * segment (32 tokens for K = 128), plus one segment's worth of per-token states per (batch, head)) grows
  * with B*H*T*K*V / 16. */
