@@ -56,6 +56,9 @@ static_assert(LDS_F32_BYTES <= 160 * 1024, "one workgroup per CU");
 // none of which depends on the state.  Waves 4-7 take the even chunks, waves 8-11 the odd ones: a group spends two
 // rounds on a chunk, so the request for its next chunk's inputs, issued when the tiles are written, has two rounds
 // to arrive.  Three buffers of tiles, chunk c in buffer c % 3.
+// WITH_O = false: the pass that only leaves the states for the backward (o_ is NULL): the three products of O, the
+// two matrices and the tile they need are left out.
+template <bool WITH_O>
 __global__ __launch_bounds__(768)
 void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restrict__ w_, const float* __restrict__ k_,
                             const float* __restrict__ v_, const float* __restrict__ a_, const float* __restrict__ b_,
@@ -181,6 +184,7 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
                     return acc;
                 };
                 if (w != 2) {
+                  if (WITH_O || w == 1) {
                     // producers 0, 1, 3: Aqk, Aak, Aqb
                     float4_t acc = gram(w == 3 ? F_BT : F_KT, w == 1 ? F_AG : F_QG);  // rows j = 4 g + e, column i = x
 #pragma unroll
@@ -190,6 +194,7 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
                     }
                     const int box = w == 0 ? 0 : (w == 3 ? 1 : 2);
                     *reinterpret_cast<float4_t*>(smem + F_BOX + box * 1024 + lane * 16) = acc;
+                  }
                 } else {
                     // producer 2: N = tril_-1(ag bt^T) and M = (I - N)^-1 = (I + N)(I + N^2)(I + N^4)(I + N^8)
                     float4_t NT_ = gram(F_BT, F_AG);   // R(N^T): lane (x = i, g): N[i][4 g + e]
@@ -316,13 +321,13 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 Y = mfma_f32(af[e], h[ct][e], Y);
-                OT = mfma_f32(h[ct][e], qf[e], OT);
+                if constexpr (WITH_O) OT = mfma_f32(h[ct][e], qf[e], OT);
             }
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             Y = mfma_f32(AakT[e], Vg[e], Y);
-            OT = mfma_f32(Vg[e], AqkT[e], OT);
+            if constexpr (WITH_O) OT = mfma_f32(Vg[e], AqkT[e], OT);
         }
         // R(SA): SA = M Y
         float4_t SA = zero4;
@@ -346,12 +351,12 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
                 for (int ct = 0; ct < 4; ++ct) h[ct] = mfma_f32(kgf[ct][e], Vg[e], h[ct]);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                OT = mfma_f32(SA[e], AqbT[e], OT);
+                if constexpr (WITH_O) OT = mfma_f32(SA[e], AqbT[e], OT);
 #pragma unroll
                 for (int ct = 0; ct < 4; ++ct) h[ct] = mfma_f32(bgf[ct][e], SA[e], h[ct]);
             }
         }
-        if (valid && o_ != nullptr)
+        if (WITH_O && valid && o_ != nullptr)
             *reinterpret_cast<float4_t*>(o_ + ((sp.tok0 + c * C16 + x) * H + hi) * NH + 16 * w + 4 * g) = OT;
         __syncthreads();
     }
@@ -371,10 +376,10 @@ hipError_t launch_fwd_chunk_f32(const SeqArgs& p, hipStream_t stream) {
         hipError_t e0 = launch_chunk_items(seq_layout(p, nullptr), nullptr, nullptr, 0, nullptr, tail_of_output(p), stream);
         if (e0 != hipSuccess) return e0;
     }
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(chunk16_f32_fwd_kernel),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(chunk16_f32_fwd_kernel<true>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, LDS_F32_BYTES);
     if (e != hipSuccess) return e;
-    chunk16_f32_fwd_kernel<<<dim3((unsigned)(p.B * p.H)), dim3(768), LDS_F32_BYTES, stream>>>(
+    chunk16_f32_fwd_kernel<true><<<dim3((unsigned)(p.B * p.H)), dim3(768), LDS_F32_BYTES, stream>>>(
         (const float*)p.r, (const float*)p.w, (const float*)p.k, (const float*)p.v, (const float*)p.a,
         (const float*)p.b, p.h0, p.h0_batch_stride, p.h0_map, p.n_state, (float*)p.o, p.ht, seq_layout(p, nullptr),
         nullptr, 0, nullptr);
@@ -385,10 +390,10 @@ hipError_t launch_fwd_chunk_f32(const SeqArgs& p, hipStream_t stream) {
 // float32 tensors, K = V = 64; seg a multiple of 16); strong (nullable): per (batch, head) whether a chunk's decay was
 // too strong for the chunk form
 hipError_t launch_fwd_chunk_f32_states(const SeqArgs& p, float* states, int seg, hipStream_t stream, int* strong) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(chunk16_f32_fwd_kernel),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(chunk16_f32_fwd_kernel<false>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, LDS_F32_BYTES);
     if (e != hipSuccess) return e;
-    chunk16_f32_fwd_kernel<<<dim3((unsigned)(p.B * p.H)), dim3(768), LDS_F32_BYTES, stream>>>(
+    chunk16_f32_fwd_kernel<false><<<dim3((unsigned)(p.B * p.H)), dim3(768), LDS_F32_BYTES, stream>>>(
         (const float*)p.r, (const float*)p.w, (const float*)p.k, (const float*)p.v, (const float*)p.a,
         (const float*)p.b, p.h0, p.h0_batch_stride, nullptr, 0, nullptr, nullptr, seq_layout(p, nullptr), states, seg,
         strong);

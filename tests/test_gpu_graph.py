@@ -147,6 +147,35 @@ def test_backward_under_graph_replay(device):
             assert torch.equal(a_, b_)
 
 
+def test_float32_backward_under_graph_replay(device):
+    """The chunked float32 backward (four launches) captured once; the replays see ordinary decays, then decays too
+    strong for the chunk form (the token-by-token kernel takes the call inside the same graph), then ordinary ones
+    again: every replay equals the eager call on the same inputs."""
+    B, T, H = 2, 100, 2
+    sets = [list(make_inputs(B, T, H, 64, seed=70 + i, dtype=torch.float32)) for i in range(3)]
+    sets[1][1] = 2.0 + torch.randn(B, T, H, 64, generator=torch.Generator().manual_seed(3))
+    stat = _static(sets[0], device)
+    g = torch.Generator().manual_seed(1)
+    d_o = torch.randn(B, T, H, 64, generator=g).to(device)
+    d_s = (0.1 * torch.randn(B, H, 64, 64, generator=g)).to(device)
+    op = torch.ops.rwkv_ops_amd.rwkv7_bwd
+    op(*stat, d_o, d_s)                                                  # warm-up
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        grads_g = op(*stat, d_o, d_s)
+    for xs in sets + sets[:1]:
+        for dst, src in zip(stat, xs):
+            dst.copy_(src.to(device))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in grads_g]
+        ref = op(*stat, d_o, d_s)
+        torch.cuda.synchronize()
+        for a_, b_ in zip(got, ref):
+            assert torch.isfinite(a_).all() and torch.equal(a_, b_)
+
+
 def test_calls_overlapping_on_two_streams(device):
     """Forward calls in flight at once on two streams (one-kernel form: workgroups of both launches wait for
     their predecessors while sharing the CUs), each with its own workspace, give the results of the same
