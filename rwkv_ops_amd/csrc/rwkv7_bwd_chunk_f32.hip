@@ -43,7 +43,8 @@ enum { BOX_AAK_T = 0, BOX_M_T, BOX_AQB, BOX_M, BOX_AQK, BOX_AAK, BOX_COUNT };
 constexpr int B_EG = B_BOX + BOX_COUNT * 1024;                           // float [64]: e^G per key channel
 constexpr int B_SCR = B_EG + 256;                                        // 1 KiB: the inverting wave transposes N here
 constexpr int BBUF = B_SCR + 1024;
-constexpr int LDS_CHAIN_BYTES = 3 * BBUF;
+constexpr int B_STAGE = 3 * BBUF;                                        // per chain wave: a staging area for its part of a state
+constexpr int LDS_CHAIN_BYTES = B_STAGE + 4 * STAGE_BYTES;
 static_assert(LDS_CHAIN_BYTES <= 160 * 1024, "one workgroup per CU");
 
 // one float of a row-major tile
@@ -226,15 +227,11 @@ void chunk16_f32_bwd_chain_kernel(const float* __restrict__ r_, const float* __r
 
     // ====================================================================== the chain
     // dh: tile ct = rows 16 ct + 4 g + e of column 16 w + x (the forward kernel's layout of the state)
-    float4_t dh[4], hn[4];
+    float4_t dh[4], hn[4];                     // hn: the state before the next chunk, on its way (as it is requested)
     const int64_t rec0 = (int64_t)bh * NT;
+    float* stage = reinterpret_cast<float*>(smem_all + B_STAGE + w * STAGE_BYTES);
     auto load_state = [&](float4_t (&dst)[4], int c, int ln) {
-        const float* src = states + (rec0 + (c < 0 ? 0 : c)) * (NH * NH) + 16 * w + (ln & 15);
-        const int g = ln >> 4;
-#pragma unroll
-        for (int ct = 0; ct < 4; ++ct)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) dst[ct][e] = src[(16 * ct + 4 * g + e) * NH];
+        state_cols_request(dst, states + (rec0 + (c < 0 ? 0 : c)) * (NH * NH) + 16 * w, ln);
     };
     {
         const int x = threadIdx.x & 15, g = (threadIdx.x & 63) >> 4;
@@ -260,16 +257,9 @@ void chunk16_f32_bwd_chain_kernel(const float* __restrict__ r_, const float* __r
         const unsigned char* smem = smem_all + (q % 3) * BBUF;
         const bool valid = c * C16 + x < T;
         // dh after this chunk, for the gradient kernel: row-major [key][value]
-        {
-            float* dst = dhs + (rec0 + c) * (NH * NH) + 16 * w + x;
-#pragma unroll
-            for (int ct = 0; ct < 4; ++ct)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) dst[(16 * ct + 4 * g + e) * NH] = dh[ct][e];
-        }
+        state_cols_store(dhs + (rec0 + c) * (NH * NH) + 16 * w, dh, stage, lane);
         float4_t h[4];
-#pragma unroll
-        for (int ct = 0; ct < 4; ++ct) h[ct] = hn[ct];
+        state_cols_unpack(h, hn, stage, lane);
         load_state(hn, c - 1, lane);           // (before the first chunk: that chunk again, never used)
 
         auto box = [&](int i) { return *reinterpret_cast<const float4_t*>(smem + B_BOX + i * 1024 + lane * 16); };

@@ -33,4 +33,37 @@ __device__ __forceinline__ float4_t tile4(const unsigned char* smem, int off, in
     return *reinterpret_cast<const float4_t*>(smem + off + (row * LDF + col) * 4);
 }
 
+// A wave's 64 x 16 part of a state (four accumulator tiles: tile ct = rows 16 ct + 4 g + e of the wave's column x)
+// against row-major [key][value] global memory: lane by lane that is sixteen 4-byte accesses, so it goes through a
+// [64][LDV] staging area of the wave's own in LDS and leaves / arrives as four 16-byte accesses (row 16 i + lane / 4,
+// sixteen bytes lane % 4 of the wave's 64-byte piece of the row).
+constexpr int LDV = 20;
+constexpr int STAGE_BYTES = NH * LDV * 4;
+__device__ __forceinline__ void state_cols_store(float* __restrict__ dst, const float4_t (&t)[4], float* stage, int lane) {
+    const int x = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) stage[(16 * ct + 4 * g + e) * LDV + x] = t[ct][e];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = 16 * i + (lane >> 2), piece = 4 * (lane & 3);
+        *reinterpret_cast<float4_t*>(dst + row * NH + piece) = *reinterpret_cast<const float4_t*>(stage + row * LDV + piece);
+    }
+}
+__device__ __forceinline__ void state_cols_request(float4_t (&q)[4], const float* __restrict__ src, int lane) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[i] = *reinterpret_cast<const float4_t*>(src + (16 * i + (lane >> 2)) * NH + 4 * (lane & 3));
+}
+__device__ __forceinline__ void state_cols_unpack(float4_t (&t)[4], const float4_t (&q)[4], float* stage, int lane) {
+    const int x = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        *reinterpret_cast<float4_t*>(stage + (16 * i + (lane >> 2)) * LDV + 4 * (lane & 3)) = q[i];
+#pragma unroll
+    for (int ct = 0; ct < 4; ++ct)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) t[ct][e] = stage[(16 * ct + 4 * g + e) * LDV + x];
+}
+
 }  // namespace rwkv7
