@@ -101,6 +101,29 @@ def test_variants(device):
     assert rel_l2(got[6], ref[6]) < TOL
 
 
+def test_many_heads_and_no_upstream_gradient(device):
+    """More (batch, head) pairs than a workgroup has threads (the flags are read in a loop), with a strong chunk in the
+    last one only; and a call with neither upstream gradient, whose seven results are zero."""
+    B, T, H = 25, 20, 40
+    xs = list(make_inputs(B, T, H, N, seed=9700, dtype=torch.float32))
+    dO, dS = upstream(B, T, H, 8)
+    rc, got = run(device, xs, dO, dS)
+    rc2, ref = run(device, xs, dO, dS, entry="rwkv7_bwd_recurrent")
+    assert rc == 0 and rc2 == 0
+    for n, a_, b_ in zip(GRAD_NAMES, got, ref):
+        assert rel_l2(a_, b_) < 1e-5 and not torch.equal(a_, b_), n      # the chunk form ran
+    xs[1] = xs[1].clone()
+    xs[1][B - 1, :16, H - 1] = 2.5
+    rc, got = run(device, xs, dO, dS)
+    rc2, ref = run(device, xs, dO, dS, entry="rwkv7_bwd_recurrent")
+    for n, a_, b_ in zip(GRAD_NAMES, got, ref):
+        assert torch.equal(a_, b_), n                                    # the token-by-token kernel ran
+    rc, got = run(device, list(make_inputs(2, 50, 2, N, seed=9701, dtype=torch.float32)), None, None)
+    assert rc == 0
+    for n, a_ in zip(GRAD_NAMES, got):
+        assert float(a_.abs().max()) == 0.0, n
+
+
 @pytest.mark.parametrize("wdist", ["normal", "strong", "one_chunk"])
 def test_strong_decays_take_the_token_by_token_kernel(device, wdist):
     """A chunk whose decay is too strong for k e^{-gi} anywhere in the call: the whole call is done by the
