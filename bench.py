@@ -372,7 +372,23 @@ def main():
 
     ms_128, _ = time_gpu(fwd_128, max(10, args.steps // 10), 2, torch)
     bytes_128 = 7 * B2 * T2 * H2 * N2 * 2 + 2 * B2 * H2 * N2 * N2 * 4
-    del x128, o128, ht128
+    # its gradients come from the float32 recurrent backward (there is no chunked backward for this head size):
+    # a quarter of the sequence, on record as microseconds per token
+    T3 = T2 // 4
+    x128b = [t[:, :T3].contiguous() for t in x128[:6]]
+    g128 = [torch.empty_like(x128b[0]) for _ in range(6)]
+    dh128 = torch.empty_like(x128[6])
+    ws128_bytes = lib.rwkv7_bwd_recurrent_workspace_bytes(B2, T3, H2, N2)
+    ws128 = torch.empty(ws128_bytes, dtype=torch.uint8, device=dev)
+
+    def bwd_128():
+        rc = lib.rwkv7_bwd_recurrent(*[ptr(t) for t in x128b], ptr(x128[6]), H2 * N2 * N2, ptr(x128b[3]), ptr(ht128),
+                                     *[ptr(g) for g in g128], ptr(dh128), B2, T3, H2, N2, N2, 0, ptr(ws128),
+                                     ws128_bytes, stream)
+        assert rc == 0, rc
+
+    ms_128_bwd, _ = time_gpu(bwd_128, 3, 1, torch)
+    del x128, o128, ht128, x128b, g128, dh128, ws128
 
     # ------------------------------------------------------------------ CPU baseline (rank 0, N = 1)
     cpu = None
@@ -505,7 +521,10 @@ def main():
         "head128": {"workload": f"rwkv7_fwd, K=V=128, B={B2} T={T2} H={H2} bf16 (the chunked kernel for that head size: one "
                                 "workgroup per (batch, head), state in registers), float32 states in and out",
                     "ms": ms_128, "tokens_per_s": B2 * T2 / (ms_128 * 1e-3), "us_per_chunk": ms_128 * 1e3 / (T2 // 64),
-                    "algorithmic_bytes": bytes_128, "frac_of_hbm_peak": bytes_128 / (ms_128 * 1e-3) / HBM_PEAK},
+                    "algorithmic_bytes": bytes_128, "frac_of_hbm_peak": bytes_128 / (ms_128 * 1e-3) / HBM_PEAK,
+                    "backward": {"workload": f"rwkv7_bwd_recurrent, K=V=128, B={B2} T={T3} H={H2} bf16 (token by token in "
+                                             "float32: this head size has no chunked backward)",
+                                 "ms": ms_128_bwd, "us_per_token": ms_128_bwd * 1e3 / T3}},
         "rwkv6": {"workload": f"RWKV6 operator forward (rwkv6_fwd), B={B} T={T} H={H} bf16, float32 states in and out",
                   "ms": ms_rwkv6, "tokens_per_s": B * T / (ms_rwkv6 * 1e-3), "algorithmic_bytes": rwkv6_bytes,
                   "frac_of_hbm_peak": rwkv6_bytes / (ms_rwkv6 * 1e-3) / HBM_PEAK},
