@@ -28,10 +28,10 @@ def get_generalized_delta_rule(HEAD_SIZE: int = 64, KERNEL_TYPE: str = "hip"):
     GPU kernel names "triton" and "cuda": they all select the HIP kernels.  "native" is
     refused: this package ships no CPU or eager implementation.  The function returned takes the head
     size from its arguments: 64 has every kernel; 128 (the head size of the reference's own value test,
-    /root/reference/test_script/test_rwkv7_value.py:51) has the decode step and a float32 recurrent
-    forward, no chunked kernels and no gradients."""
+    /root/reference/test_script/test_rwkv7_value.py:51) has the decode step, a chunked bf16 forward, and
+    token-by-token float32 kernels for everything else, gradients included (no chunked backward)."""
     if int(HEAD_SIZE) not in (64, 128):
-        raise NotImplementedError(f"HEAD_SIZE={HEAD_SIZE}: head sizes 64 and 128 (forward only) are built")
+        raise NotImplementedError(f"HEAD_SIZE={HEAD_SIZE}: head sizes 64 and 128 are built")
     kt = str(KERNEL_TYPE).lower()
     if kt not in ("hip", "triton", "cuda"):
         raise NotImplementedError(

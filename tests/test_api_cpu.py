@@ -12,7 +12,7 @@ def test_facade_names():
     assert rwkv_ops_amd.rwkv7_op is rwkv_ops_amd.generalized_delta_rule
     assert rwkv_ops_amd.RWKV7_USE_KERNEL is True
     assert rwkv_ops_amd.get_generalized_delta_rule(KERNEL_TYPE="triton")[1] is True
-    assert rwkv_ops_amd.get_generalized_delta_rule(128)[0] is rwkv_ops_amd.generalized_delta_rule   # forward only
+    assert rwkv_ops_amd.get_generalized_delta_rule(128)[0] is rwkv_ops_amd.generalized_delta_rule
     with pytest.raises(NotImplementedError):
         rwkv_ops_amd.get_generalized_delta_rule(256)
     with pytest.raises(NotImplementedError):
