@@ -254,7 +254,8 @@ int rwkv7_bwd_recurrent(const void* r, const void* w, const void* k, const void*
  * each sequence's own first token, so the result for a sequence does not depend on
  * where it lies in the packed row.  The lengths never travel to the host: grids and
  * workspaces are sized for the most chunks T_total tokens in n_seq sequences can have
- * (T_total / 64 + n_seq per head).  bf16 and, forward only, f32. */
+ * (T_total / 64 + n_seq per head).  bf16 and f32 (f32: the chunked float32 kernels on 16-token chunks,
+ * T_total / 16 + n_seq records per head in the backward's workspace; the forward takes none). */
 size_t rwkv7_fwd_varlen_workspace_bytes(int n_seq, int T_total, int H, int dtype);
 int rwkv7_fwd_varlen(const void* r, const void* w, const void* k, const void* v,
                      const void* a, const void* b,

@@ -397,7 +397,9 @@ int rwkv7_fwd_varlen(const void* r, const void* w, const void* k, const void* v,
 }
 
 size_t rwkv7_bwd_varlen_workspace_bytes(int n_seq, int T_total, int H, int dtype) {
-    if (dtype != RWKV7_DTYPE_BF16 || n_seq < 1 || T_total < 1 || H < 1) return 0;
+    if (n_seq < 1 || T_total < 1 || H < 1) return 0;
+    if (dtype == RWKV7_DTYPE_F32) return rwkv7::bwd_chunk_f32_workspace_bytes(n_seq, T_total, H, true);
+    if (dtype != RWKV7_DTYPE_BF16) return 0;
     return rwkv7::bwd_chunk_workspace_bytes(n_seq, T_total, H, true);
 }
 
@@ -407,7 +409,8 @@ int rwkv7_bwd_varlen(const void* r, const void* w, const void* k, const void* v,
                      void* dr, void* dw, void* dk, void* dv, void* da, void* db, float* dh0,
                      int T_total, int H, int K, int V, int dtype, void* ws, size_t ws_bytes, void* stream)
 {
-    if (dtype == RWKV7_DTYPE_F32) return RWKV7_ERR_UNSUPPORTED;
+    // float32 tensors (K = V = 64): the chunked float32 backward over the packed sequences
+    const bool f32 = dtype == RWKV7_DTYPE_F32 && K == 64 && V == 64;
     int rc = check_seq(r, w, k, v, a, b, h0, h0_batch_stride, dr, nullptr, 1, T_total, H, K, V, dtype);
     if (rc != RWKV7_OK) return rc;
     rc = check_varlen(cu_seqlens, n_seq, T_total, H);
@@ -416,7 +419,8 @@ int rwkv7_bwd_varlen(const void* r, const void* w, const void* k, const void* v,
     if (!aligned16(d_o) || !aligned16(d_ht) || !aligned16(dw) || !aligned16(dk) || !aligned16(dv) ||
         !aligned16(da) || !aligned16(db) || !aligned16(dh0))
         return RWKV7_ERR_ALIGNMENT;
-    const size_t need = rwkv7::bwd_chunk_workspace_bytes(n_seq, T_total, H, true);
+    const size_t need = f32 ? rwkv7::bwd_chunk_f32_workspace_bytes(n_seq, T_total, H, true)
+                            : rwkv7::bwd_chunk_workspace_bytes(n_seq, T_total, H, true);
     if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return RWKV7_ERR_WORKSPACE;
     rwkv7::BwdArgs p;
     p.r = r; p.w = w; p.k = k; p.v = v; p.a = a; p.b = b;
@@ -424,6 +428,7 @@ int rwkv7_bwd_varlen(const void* r, const void* w, const void* k, const void* v,
     p.dO = d_o; p.dht = d_ht;
     p.dr = dr; p.dw = dw; p.dk = dk; p.dv = dv; p.da = da; p.db = db; p.dh0 = dh0;
     p.B = n_seq; p.T = T_total; p.H = H; p.dtype = dtype; p.cu = cu_seqlens;
+    if (f32) return (int)rwkv7::launch_bwd_chunk_f32(p, ws, static_cast<hipStream_t>(stream));
     return (int)rwkv7::launch_bwd_chunk(p, ws, static_cast<hipStream_t>(stream));
 }
 

@@ -91,17 +91,28 @@ void chunk16_f32_bwd_chain_kernel(const float* __restrict__ r_, const float* __r
                                   const float* __restrict__ do_, const float* __restrict__ dht,
                                   const float* __restrict__ states, const int* __restrict__ strong_flags,
                                   float* __restrict__ dhs, float* __restrict__ sa_ws, float* __restrict__ dy_ws,
-                                  float* __restrict__ dv_, float* __restrict__ dh0, int B, int T, int H)
+                                  float* __restrict__ dv_, float* __restrict__ dh0, SeqLayout L)
 {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_all[];
-    if (any_strong(strong_flags, B * H)) return;
+    const int H = L.H;
+    if (any_strong(strong_flags, L.B * H)) return;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int w = wave & 3;
     const bool producer = wave >= 4;
     const int bh = blockIdx.x, hi = bh % H, bi = bh / H;
-    const int NT = (T + C16 - 1) / C16;
-    const int64_t tok0 = (int64_t)bi * T;
+    const SeqSpan sp = seq_span(L, bi);
+    const int T = sp.len, NT = (T + C16 - 1) / C16;
+    const int64_t tok0 = sp.tok0;
     const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+    if (NT == 0) {                             // a sequence without tokens: the adjoint passes through
+        if (!producer && dh0 != nullptr) {
+            const int x = threadIdx.x & 15, g = (threadIdx.x & 63) >> 4;
+            float* dst = dh0 + (int64_t)bh * (NH * NH) + 16 * w + x;
+            const float* src = dht == nullptr ? nullptr : dht + (int64_t)bh * (NH * NH) + 16 * w + x;
+            for (int i = 0; i < 16; ++i) dst[(4 * i + g) * NH] = src ? src[(4 * i + g) * NH] : 0.f;
+        }
+        return;
+    }
     const int ROUNDS = NT + 2;
 
     if (producer) {
@@ -228,10 +239,10 @@ void chunk16_f32_bwd_chain_kernel(const float* __restrict__ r_, const float* __r
     // ====================================================================== the chain
     // dh: tile ct = rows 16 ct + 4 g + e of column 16 w + x (the forward kernel's layout of the state)
     float4_t dh[4], hn[4];                     // hn: the state before the next chunk, on its way (as it is requested)
-    const int64_t rec0 = (int64_t)bh * NT;
+    const ChunkRecords record = f32_chunk_records(L, sp, bi, hi, NT);
     float* stage = reinterpret_cast<float*>(smem_all + B_STAGE + w * STAGE_BYTES);
     auto load_state = [&](float4_t (&dst)[4], int c, int ln) {
-        state_cols_request(dst, states + (rec0 + (c < 0 ? 0 : c)) * (NH * NH) + 16 * w, ln);
+        state_cols_request(dst, states + record(c < 0 ? 0 : c) * (NH * NH) + 16 * w, ln);
     };
     {
         const int x = threadIdx.x & 15, g = (threadIdx.x & 63) >> 4;
@@ -257,7 +268,7 @@ void chunk16_f32_bwd_chain_kernel(const float* __restrict__ r_, const float* __r
         const unsigned char* smem = smem_all + (q % 3) * BBUF;
         const bool valid = c * C16 + x < T;
         // dh after this chunk, for the gradient kernel: row-major [key][value]
-        state_cols_store(dhs + (rec0 + c) * (NH * NH) + 16 * w, dh, stage, lane);
+        state_cols_store(dhs + record(c) * (NH * NH) + 16 * w, dh, stage, lane);
         float4_t h[4];
         state_cols_unpack(h, hn, stage, lane);
         load_state(hn, c - 1, lane);           // (before the first chunk: that chunk again, never used)
@@ -328,7 +339,7 @@ void chunk16_f32_bwd_chain_kernel(const float* __restrict__ r_, const float* __r
                     dh[ct] = mfma_f32(tile1(smem, B_AG, 4 * g + e, 16 * ct + x), dY[e], dh[ct]);
         }
         {
-            const int64_t rec = rec0 + c;
+            const int64_t rec = record(c);
             *reinterpret_cast<float4_t*>(sa_ws + rec * (C16 * NH) + x * NH + 16 * w + 4 * g) = SAT;
             *reinterpret_cast<float4_t*>(dy_ws + rec * (C16 * NH) + x * NH + 16 * w + 4 * g) = dYT;
             if (valid)
@@ -368,21 +379,42 @@ void chunk16_f32_bwd_grad_kernel(const float* __restrict__ r_, const float* __re
                                  const int* __restrict__ strong_flags, const float* __restrict__ dhs,
                                  const float* __restrict__ sa_ws, const float* __restrict__ dy_ws,
                                  float* __restrict__ dr_, float* __restrict__ dw_, float* __restrict__ dk_,
-                                 float* __restrict__ da_, float* __restrict__ db_, int B, int T, int H)
+                                 float* __restrict__ da_, float* __restrict__ db_, SeqLayout L)
 {
     __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_GRAD_BYTES];
     // (the forward pass's flags are asked for now and looked at only before the stores: nothing here waits for them)
+    const int H = L.H;
     int flagged = 0;
-    for (int i = threadIdx.x; i < B * H; i += 256) flagged |= strong_flags[i];
+    for (int i = threadIdx.x; i < L.B * H; i += 256) flagged |= strong_flags[i];
     const int lane = threadIdx.x & 63;
     const int w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int x = lane & 15, g = lane >> 4;
-    const int NT = (T + C16 - 1) / C16;
-    const int c = blockIdx.x % NT, bh = blockIdx.x / NT, hi = bh % H, bi = bh / H;
-    const int64_t rec = (int64_t)bh * NT + c;
+    int c, bi, hi;
+    if (L.cu == nullptr) {                     // dense: workgroup (b H + h) NT + c
+        const int nt = (L.T + C16 - 1) / C16;
+        c = blockIdx.x % nt;
+        const int bh = blockIdx.x / nt;
+        hi = bh % H; bi = bh / H;
+    } else {
+        // packed: workgroup slot H + h; the slot's sequence is the last one that starts at or before it (slots of a
+        // sequence start at (first row / 16) + its index, which grows with the index), found by bisection
+        const int slot = blockIdx.x / H;
+        hi = blockIdx.x % H;
+        int lo = 0, up = L.B - 1;
+        while (lo < up) {
+            const int mid = (lo + up + 1) >> 1;
+            if ((int)(seq_span(L, mid).tok0 >> 4) + mid <= slot) lo = mid; else up = mid - 1;
+        }
+        bi = lo;
+        c = slot - ((int)(seq_span(L, bi).tok0 >> 4) + bi);
+    }
+    const SeqSpan sp = seq_span(L, bi);
+    const int T = sp.len, NT = (T + C16 - 1) / C16;
+    if (c < 0 || c >= NT) return;              // (packed: a slot between two sequences)
+    const int64_t rec = f32_chunk_records(L, sp, bi, hi, NT)(c);
     const int t = c * C16 + x;
     const bool valid = t < T;
-    const int64_t row = (((int64_t)bi * T + (valid ? t : T - 1)) * H + hi) * NH;
+    const int64_t row = ((sp.tok0 + (valid ? t : T - 1)) * H + hi) * NH;
     const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 
     // ---- this wave's channels of the inputs, scaled, and four of the scaled operands transposed:
@@ -535,7 +567,7 @@ void chunk16_f32_bwd_grad_kernel(const float* __restrict__ r_, const float* __re
     {
         const int tok = 4 * w + g, piece = 4 * x, ts = c * C16 + tok;
         if (ts < T && !strong) {
-            const int64_t o = (((int64_t)bi * T + ts) * H + hi) * NH + piece;
+            const int64_t o = ((sp.tok0 + ts) * H + hi) * NH + piece;
             *reinterpret_cast<float4_t*>(dr_ + o) = tile4(smem, G_V, tok, piece);
             *reinterpret_cast<float4_t*>(dw_ + o) = tile4(smem, G_DO, tok, piece);
             *reinterpret_cast<float4_t*>(dk_ + o) = tile4(smem, G_SA, tok, piece);
@@ -545,44 +577,65 @@ void chunk16_f32_bwd_grad_kernel(const float* __restrict__ r_, const float* __re
     }
 }
 
-// Workspace: the state before every chunk, dh after every chunk, SA and dY of every chunk, the token-by-token
-// kernel's per-workgroup scratch (64 states), one flag per (batch, head).
-size_t bwd_chunk_f32_workspace_bytes(int B, int T, int H) {
-    const size_t BH = (size_t)B * H, NT = (size_t)(T + C16 - 1) / C16;
+// Workspace: per record (one per 16-token chunk and head; packed sequences: (T_total / 16 + n_seq) H of them) the state
+// before the chunk, dh after it, SA and dY; the token-by-token kernel's scratch areas (64 states each: one per
+// (batch, head), at most WALK_MAX_GRID with packed sequences); one flag per (sequence, head).
+namespace {
+size_t f32_records(int B, int T, int H, bool varlen) {
+    return varlen ? ((size_t)(T >> 4) + B) * H : (size_t)B * H * ((T + C16 - 1) / C16);
+}
+size_t walk_areas(int B, int H, bool varlen) {
+    const size_t bh = (size_t)B * H;
+    return varlen && bh > (size_t)WALK_MAX_GRID ? (size_t)WALK_MAX_GRID : bh;
+}
+}  // namespace
+
+size_t bwd_chunk_f32_workspace_bytes(int B, int T, int H, bool varlen) {
     const size_t per_chunk = (size_t)(2 * NH * NH + 2 * C16 * NH) * 4;
-    return BH * NT * per_chunk + BH * 64 * (size_t)(NH * NH) * 4 + ((BH * 4 + 255) & ~(size_t)255);
+    return f32_records(B, T, H, varlen) * per_chunk + walk_areas(B, H, varlen) * 64 * (size_t)(NH * NH) * 4 +
+           (((size_t)B * H * 4 + 255) & ~(size_t)255);
 }
 
 hipError_t launch_bwd_chunk_f32(const BwdArgs& p, void* ws, hipStream_t stream) {
-    const size_t BH = (size_t)p.B * p.H, NT = (size_t)(p.T + C16 - 1) / C16;
+    const bool varlen = p.cu != nullptr;
+    const size_t BH = (size_t)p.B * p.H, NR = f32_records(p.B, p.T, p.H, varlen);
     float* states = static_cast<float*>(ws);
-    float* dhs = states + BH * NT * (NH * NH);
-    float* sa = dhs + BH * NT * (NH * NH);
-    float* dy = sa + BH * NT * (C16 * NH);
-    float* scratch = dy + BH * NT * (C16 * NH);
-    int* flags = reinterpret_cast<int*>(scratch + BH * 64 * (size_t)(NH * NH));
+    float* dhs = states + NR * (NH * NH);
+    float* sa = dhs + NR * (NH * NH);
+    float* dy = sa + NR * (C16 * NH);
+    float* scratch = dy + NR * (C16 * NH);
+    int* flags = reinterpret_cast<int*>(scratch + walk_areas(p.B, p.H, varlen) * 64 * (size_t)(NH * NH));
     // launch 1: the forward once more, leaving the state before every chunk and the flags
     SeqArgs f{};
     f.r = p.r; f.w = p.w; f.k = p.k; f.v = p.v; f.a = p.a; f.b = p.b;
     f.h0 = p.h0; f.h0_batch_stride = p.h0 ? p.h0_batch_stride : 0;
-    f.B = p.B; f.T = p.T; f.H = p.H; f.N = NH; f.dtype = p.dtype;
-    hipError_t e = launch_fwd_chunk_f32_states(f, states, C16, stream, flags);
+    f.B = p.B; f.T = p.T; f.H = p.H; f.N = NH; f.dtype = p.dtype; f.cu = p.cu;
+    const SeqLayout L = seq_layout(f, nullptr);
+    hipError_t e;
+    if (varlen) {                      // rows of the gradients behind the last sequence
+        TailFill tail;
+        tail.p[0] = p.dr; tail.p[1] = p.dw; tail.p[2] = p.dk; tail.p[3] = p.dv; tail.p[4] = p.da; tail.p[5] = p.db;
+        tail.n = 6; tail.row_bytes = (int64_t)p.H * NH * 4;
+        e = launch_chunk_items(L, nullptr, nullptr, 0, nullptr, tail, stream);
+        if (e != hipSuccess) return e;
+    }
+    e = launch_fwd_chunk_f32_states(f, states, C16, stream, flags);
     if (e != hipSuccess) return e;
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(chunk16_f32_bwd_chain_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_CHAIN_BYTES);
     if (e != hipSuccess) return e;
     chunk16_f32_bwd_chain_kernel<<<dim3((unsigned)BH), dim3(768), LDS_CHAIN_BYTES, stream>>>(
         (const float*)p.r, (const float*)p.w, (const float*)p.k, (const float*)p.v, (const float*)p.a,
-        (const float*)p.b, (const float*)p.dO, p.dht, states, flags, dhs, sa, dy, (float*)p.dv, p.dh0, p.B, p.T, p.H);
+        (const float*)p.b, (const float*)p.dO, p.dht, states, flags, dhs, sa, dy, (float*)p.dv, p.dh0, L);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    chunk16_f32_bwd_grad_kernel<<<dim3((unsigned)(BH * NT)), dim3(256), 0, stream>>>(
+    chunk16_f32_bwd_grad_kernel<<<dim3((unsigned)NR), dim3(256), 0, stream>>>(
         (const float*)p.r, (const float*)p.w, (const float*)p.k, (const float*)p.v, (const float*)p.a,
         (const float*)p.b, (const float*)p.dO, states, flags, dhs, sa, dy, (float*)p.dr, (float*)p.dw, (float*)p.dk,
-        (float*)p.da, (float*)p.db, p.B, p.T, p.H);
+        (float*)p.da, (float*)p.db, L);
     e = hipGetLastError();
     if (e != hipSuccess) return e;
-    // strong decays somewhere: the two kernels above have returned at once, this one does the call
+    // strong decays somewhere: the two kernels above have returned at once / stored nothing, this one does the call
     return launch_bwd_recurrent_walk_f32(p, states, scratch, flags, (int)BH, stream);
 }
 

@@ -75,11 +75,16 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
                           const T* __restrict__ d_o, const float* __restrict__ d_ht,
                           const float* __restrict__ ckpt, float* __restrict__ scratch,
                           T* __restrict__ dr, T* __restrict__ dw, T* __restrict__ dk, T* __restrict__ dv,
-                          T* __restrict__ da, T* __restrict__ db, float* __restrict__ dh0, int T_len, int H,
-                          int ckpt_per_head, int ckpt_step, const int* __restrict__ run_if_any, int n_flags)
+                          T* __restrict__ da, T* __restrict__ db, float* __restrict__ dh0, int T_rows, int H,
+                          int ckpt_per_head, int ckpt_step, const int* __restrict__ run_if_any, int n_flags,
+                          const int* __restrict__ cu, int n_bh)
 {
     // ckpt: the state before token SEG * s is record ckpt_step * s of this head's ckpt_per_head records.
     // run_if_any (nullable): n_flags integers; the kernel runs only when one of them is not zero.
+    // cu (nullable): packed sequences -- cumulative lengths of the n_bh / H sequences in one row of T_rows tokens;
+    // the checkpoints are then the records of the chunked float32 backward (sequence b, segment s: record
+    // ((first row / 16) + b + 4 s) H + h).  The grid may be smaller than n_bh: a workgroup takes every gridDim.x-th
+    // (sequence, head) and owns one scratch area.
     constexpr int CPW = RecShape<N>::CPW, SEG = RecShape<N>::SEG;
     constexpr int VQ = CPW / 4;                  // lanes across a wave's columns, four columns each
     constexpr int ROWS = N / (64 / VQ);          // state rows per lane
@@ -103,16 +108,27 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
     }
     const int lane = tid & 63;
     const int wave = tid >> 6;                   // which CPW value columns
-    const int bh = blockIdx.x, hi = bh % H;
     const int ks = lane / VQ, vq = lane % VQ;
     const int col0 = CPW * wave + 4 * vq;        // this lane's four value columns
     const int row0 = ROWS * ks;                  // this lane's first state row
     const int tile = row0 * N + col0;
     const int64_t step = (int64_t)H * N;
-    const int64_t base = ((int64_t)(bh / H) * T_len * H + hi) * N;
+    float* my_scr = scratch + (int64_t)blockIdx.x * SEG * (N * N);
+  for (int bh = blockIdx.x; bh < n_bh; bh += gridDim.x) {
+    const int hi = bh % H, bi = bh / H;
+    int64_t tok0 = (int64_t)bi * T_rows;
+    int T_len = T_rows;
+    if (cu != nullptr) {
+        int s0 = load_table(cu + bi), e0 = load_table(cu + bi + 1);
+        s0 = s0 < 0 ? 0 : (s0 > T_rows ? T_rows : s0);
+        e0 = e0 < s0 ? s0 : (e0 > T_rows ? T_rows : e0);
+        tok0 = s0; T_len = e0 - s0;
+    }
+    const int64_t base = (tok0 * H + hi) * N;
     const int nseg = (T_len + SEG - 1) / SEG;
-    const float* my_ckpt = ckpt + (int64_t)bh * ckpt_per_head * (N * N);
-    float* my_scr = scratch + (int64_t)bh * SEG * (N * N);
+    const float* my_ckpt = cu != nullptr ? ckpt + (((tok0 >> 4) + bi) * H + hi) * (int64_t)(N * N)
+                                         : ckpt + (int64_t)bh * ckpt_per_head * (N * N);
+    const int64_t ckpt_stride = cu != nullptr ? (int64_t)4 * H * (N * N) : (int64_t)ckpt_step * (N * N);
 
     // one block of per-token vectors -> LDS as float (w as the decay d, and as dfac = dd/dw = -exp(w) d)
     auto stage_block = [&](int t0, int nt, bool reverse_pass) {
@@ -174,7 +190,7 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
         // ---- the segment forward once more: the state before each token -> scratch, sa -> LDS
         {
             float4_t s[ROWS];
-            const float* src = my_ckpt + (int64_t)seg * ckpt_step * (N * N) + tile;
+            const float* src = my_ckpt + (int64_t)seg * ckpt_stride + tile;
 #pragma unroll
             for (int i = 0; i < ROWS; ++i) s[i] = *reinterpret_cast<const float4_t*>(src + i * N);
             for (int t0 = 0; t0 < slen; t0 += RB_TB) {
@@ -278,6 +294,8 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
 #pragma unroll
         for (int i = 0; i < ROWS; ++i) *reinterpret_cast<float4_t*>(dst + i * N) = Hd[i];
     }
+    __syncthreads();                             // (the next (sequence, head) of this workgroup reuses the LDS areas)
+  }
 }
 
 namespace {
@@ -287,25 +305,30 @@ template <int N> constexpr size_t rec_lds_bytes() {
 
 template <typename T, int N>
 hipError_t launch_bwd_rec_t(const BwdArgs& p, const float* ckpt, float* scratch, hipStream_t stream,
-                            int ckpt_per_head = 0, int ckpt_step = 1, const int* run_if_any = nullptr, int n_flags = 0) {
+                            int ckpt_per_head = 0, int ckpt_step = 1, const int* run_if_any = nullptr, int n_flags = 0,
+                            int max_grid = 0) {
     if (ckpt_per_head == 0) ckpt_per_head = (p.T + RecShape<N>::SEG - 1) / RecShape<N>::SEG;
+    const int n_bh = p.B * p.H;
+    const int grid = max_grid > 0 && n_bh > max_grid ? max_grid : n_bh;
     constexpr size_t lds = rec_lds_bytes<N>();
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_recurrent_kernel<T, N>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
-    bwd_recurrent_kernel<T, N><<<dim3((unsigned)(p.B * p.H)), dim3(256), lds, stream>>>(
+    bwd_recurrent_kernel<T, N><<<dim3((unsigned)grid), dim3(256), lds, stream>>>(
         (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, (const T*)p.a, (const T*)p.b,
         (const T*)p.dO, p.dht, ckpt, scratch, (T*)p.dr, (T*)p.dw, (T*)p.dk, (T*)p.dv, (T*)p.da, (T*)p.db,
-        p.dh0, p.T, p.H, ckpt_per_head, ckpt_step, run_if_any, n_flags);
+        p.dh0, p.T, p.H, ckpt_per_head, ckpt_step, run_if_any, n_flags, p.cu, n_bh);
     return hipGetLastError();
 }
 }  // namespace
 
-// the walk alone, for float32 tensors at K = V = 64, over states stored every 16 tokens (record 4 s = the state
-// before token 64 s); it runs only when one of the n_flags integers at run_if_any is not zero
+// the walk alone, for float32 tensors at K = V = 64, over states stored every 16 tokens (dense: record 4 s of a head
+// = the state before token 64 s; packed (p.cu): the records of the chunked float32 backward); it runs only when one of
+// the n_flags integers at run_if_any is not zero; at most WALK_MAX_GRID workgroups, each with a scratch area of 64 states
 hipError_t launch_bwd_recurrent_walk_f32(const BwdArgs& p, const float* states16, float* scratch,
                                          const int* run_if_any, int n_flags, hipStream_t stream) {
-    return launch_bwd_rec_t<float, 64>(p, states16, scratch, stream, (p.T + 15) / 16, 4, run_if_any, n_flags);
+    return launch_bwd_rec_t<float, 64>(p, states16, scratch, stream, (p.T + 15) / 16, 4, run_if_any, n_flags,
+                                       p.cu != nullptr ? WALK_MAX_GRID : 0);
 }
 
 hipError_t launch_bwd_recurrent(const BwdArgs& p, int N, void* ws, hipStream_t stream) {

@@ -2,6 +2,7 @@
 // layouts are described at the top of rwkv7_fwd_chunk_f32.hip.
 #pragma once
 #include "rwkv7_chunk.h"
+#include "rwkv7_common.h"
 
 namespace rwkv7 {
 
@@ -64,6 +65,19 @@ __device__ __forceinline__ void state_cols_unpack(float4_t (&t)[4], const float4
     for (int ct = 0; ct < 4; ++ct)
 #pragma unroll
         for (int e = 0; e < 4; ++e) t[ct][e] = stage[(16 * ct + 4 * g + e) * LDV + x];
+}
+
+// Workspace records of the float32 backward, one per 16-token chunk and head.  Dense batches: record
+// (b H + h) NT + c.  Packed sequences: sequence b owns the slots from (first row / 16) + b on -- at most
+// len / 16 + 1 of them, never overlapping the next sequence's -- and the record of its chunk c is (slot + c) H + h;
+// (T_total / 16 + n_seq) H records in all.
+struct ChunkRecords {
+    int64_t first; int step;           // record of chunk c: first + c * step
+    __device__ __forceinline__ int64_t operator()(int c) const { return first + (int64_t)c * step; }
+};
+__device__ __forceinline__ ChunkRecords f32_chunk_records(const SeqLayout& L, const SeqSpan& sp, int bi, int hi, int nt) {
+    if (L.cu == nullptr) return ChunkRecords{((int64_t)bi * L.H + hi) * nt, 1};
+    return ChunkRecords{((sp.tok0 >> 4) + bi) * L.H + hi, L.H};
 }
 
 }  // namespace rwkv7

@@ -66,8 +66,9 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
                             int n_state, float* __restrict__ o_, float* __restrict__ ht, SeqLayout L,
                             float* __restrict__ seg_states, int seg, int* __restrict__ strong_out)
 {
-    // seg_states (dense batches): the state BEFORE token t is stored for every t that is a multiple of `seg` (a
-    // multiple of 16), [workgroup][t / seg][64][64]: what the backward kernels restart from.  o_ may then be NULL.
+    // seg_states: the state BEFORE token t is stored for every t that is a multiple of `seg` (a multiple of 16),
+    // dense batches [workgroup][t / seg][64][64], packed sequences (seg = 16 only) the records of f32_chunk_records: what the
+    // backward kernels restart from.  o_ may then be NULL.
     // strong_out (nullable): one integer per workgroup, 1 when a chunk of its sequence was walked token by token.
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_all[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -257,6 +258,10 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
     }
     __syncthreads();                           // rounds 0 and 1: the first chunk is on its way
     __syncthreads();
+    // where the states go: dense [workgroup][t / seg], packed the records of the float32 backward (seg = 16)
+    const ChunkRecords packed_recs = f32_chunk_records(L, sp, bi, hi, NT);
+    const int64_t seg_first = L.cu != nullptr ? packed_recs.first : (int64_t)bh * ((T + seg - 1) / seg);
+    const int seg_step = L.cu != nullptr ? packed_recs.step : 1;
     bool any_strong = false;
     for (int c = 0; c < NT; ++c) {             // round c + 2
         int lane = threadIdx.x & 63;
@@ -265,7 +270,7 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
         const unsigned char* smem = smem_all + (c % 3) * BUF_BYTES;
         const bool valid = c * C16 + x < T;
         if (seg_states != nullptr && (c * C16) % seg == 0) {
-            float* dst = seg_states + ((int64_t)bh * ((T + seg - 1) / seg) + (c * C16) / seg) * (NH * NH) + 16 * w + x;
+            float* dst = seg_states + (seg_first + (int64_t)((c * C16) / seg) * seg_step) * (NH * NH) + 16 * w + x;
 #pragma unroll
             for (int ct = 0; ct < 4; ++ct)
 #pragma unroll
@@ -386,9 +391,9 @@ hipError_t launch_fwd_chunk_f32(const SeqArgs& p, hipStream_t stream) {
     return hipGetLastError();
 }
 
-// the forward without outputs, storing the state at the start of every segment of `seg` tokens (dense batches,
-// float32 tensors, K = V = 64; seg a multiple of 16); strong (nullable): per (batch, head) whether a chunk's decay was
-// too strong for the chunk form
+// the forward without outputs, storing the state at the start of every segment of `seg` tokens (float32 tensors,
+// K = V = 64; seg a multiple of 16, dense batches, or 16 with packed sequences (p.cu)); strong (nullable): per
+// (batch, head) whether a chunk's decay was too strong for the chunk form
 hipError_t launch_fwd_chunk_f32_states(const SeqArgs& p, float* states, int seg, hipStream_t stream, int* strong) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(chunk16_f32_fwd_kernel<false>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, LDS_F32_BYTES);
@@ -397,6 +402,7 @@ hipError_t launch_fwd_chunk_f32_states(const SeqArgs& p, float* states, int seg,
         (const float*)p.r, (const float*)p.w, (const float*)p.k, (const float*)p.v, (const float*)p.a,
         (const float*)p.b, p.h0, p.h0_batch_stride, nullptr, 0, nullptr, nullptr, seq_layout(p, nullptr), states, seg,
         strong);
+    static_assert(C16 == 16, "packed records are per 16-token chunk");
     return hipGetLastError();
 }
 

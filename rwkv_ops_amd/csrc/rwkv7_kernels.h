@@ -90,11 +90,12 @@ hipError_t launch_bwd_recurrent(const BwdArgs& p, int N, void* ws, hipStream_t s
 hipError_t launch_fwd_recurrent_states(const SeqArgs& p, float* states, int seg, hipStream_t stream);
 // its second launch alone, float32 tensors at K = V = 64, over states stored every 16 tokens; runs only when one of
 // the n_flags integers at run_if_any is not zero
+constexpr int WALK_MAX_GRID = 1024;     // workgroups of the walk over packed sequences (each owns 1 MiB of scratch)
 hipError_t launch_bwd_recurrent_walk_f32(const BwdArgs& p, const float* states16, float* scratch,
                                          const int* run_if_any, int n_flags, hipStream_t stream);
-// chunked float32 backward (float32 tensors, K = V = 64, dense batches) on the float32 matrix cores;
+// chunked float32 backward (float32 tensors, K = V = 64; dense batches or packed sequences, p.cu) on the float32 matrix cores;
 // ws holds bwd_chunk_f32_workspace_bytes(B, T, H) bytes, 256-byte aligned
-size_t bwd_chunk_f32_workspace_bytes(int B, int T, int H);
+size_t bwd_chunk_f32_workspace_bytes(int B, int T, int H, bool varlen = false);
 hipError_t launch_bwd_chunk_f32(const BwdArgs& p, void* ws, hipStream_t stream);
 // RWKV6 backward (stateless call, bf16): runs the RWKV7 backward kernels on operands read one token ahead
 // plus an epilogue for the bonus term; du is float32 [H, 64]

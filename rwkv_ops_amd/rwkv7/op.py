@@ -290,7 +290,7 @@ def rwkv7_bwd_varlen(r: torch.Tensor, w: torch.Tensor, k: torch.Tensor, v: torch
                      d_o: Optional[torch.Tensor], d_ht: Optional[torch.Tensor], cu: torch.Tensor
                      ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
                                 torch.Tensor, torch.Tensor]:
-    """Gradients of ``rwkv7_fwd_varlen`` (bf16): ``(dr, dw, dk, dv, da, db, dh0)``, ``dh0`` float32
+    """Gradients of ``rwkv7_fwd_varlen`` (bf16 or float32): ``(dr, dw, dk, dv, da, db, dh0)``, ``dh0`` float32
     ``[n_seq, H, 64, 64]``.  Rows of the packed batch that belong to no sequence get zero gradients."""
     lib = _lib.load()
     _, T, H, N = r.shape
@@ -325,8 +325,11 @@ def _fwd_varlen_setup_context(ctx, inputs, output):
 def _fwd_varlen_backward(ctx, d_o, d_ht):
     r, w, k, v, a, b, h0, cu = ctx.saved_tensors
     dt = r.dtype
-    cast = (lambda t: t.to(torch.bfloat16)) if dt != torch.bfloat16 else (lambda t: t)
-    d_o_c = None if d_o is None else cast(d_o).contiguous()
+    # float32 rows at head size 64 keep float32 (the chunked float32 backward); float16 rows are rounded to bf16 as in
+    # the dense call
+    exact = dt == torch.bfloat16 or (dt == torch.float32 and r.shape[-1] == HEAD_SIZE)
+    cast = (lambda t: t) if exact else (lambda t: t.to(torch.bfloat16))
+    d_o_c = None if d_o is None else cast(d_o.to(dt)).contiguous()
     d_ht_c = None
     if ctx.want_state and d_ht is not None and d_ht.numel() > 0:
         d_ht_c = d_ht.to(torch.float32).contiguous()

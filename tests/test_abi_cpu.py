@@ -102,7 +102,13 @@ def test_varlen_argument_errors_do_not_launch():
     assert lib.rwkv7_fwd_varlen_workspace_bytes(64, T, H, 0) < 64 * H * 40000   # one-kernel form: no per-chunk records
     rc = lib.rwkv7_bwd_varlen(*[0x1000] * 6, 0x3000, 2, None, 0, None, None, *[0x1000] * 6, None,
                               100, 2, 64, 64, 1, None, 0, None)
-    assert rc == -8                                      # float32 backward is not built
+    assert rc == -6                                      # float32 rows: the chunked float32 backward, which needs
+    # 40 KiB per 16 tokens (T / 16 + n_seq records per head) and 1 MiB per sequence-head, up to 1024 of them
+    assert lib.rwkv7_bwd_varlen_workspace_bytes(n_seq, T, H, 1) >= (T // 16 + n_seq) * H * 40960 + n_seq * H * (1 << 20)
+    assert lib.rwkv7_bwd_varlen_workspace_bytes(2000, 20000, 4, 1) < (20000 // 16 + 2000) * 4 * 40960 + 1025 * (1 << 20)
+    rc = lib.rwkv7_bwd_varlen(*[0x1000] * 6, 0x3000, 2, None, 0, None, None, *[0x1000] * 6, None,
+                              100, 2, 128, 128, 1, None, 0, None)
+    assert rc == -3                                      # ... at head size 64 only
     rc = lib.rwkv7_bwd_varlen(*[0x1000] * 6, None, 2, None, 0, None, None, *[0x1000] * 6, None,
                               100, 2, 64, 64, 0, None, 0, None)
     assert rc == -1

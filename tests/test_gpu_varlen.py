@@ -191,6 +191,58 @@ def test_varlen_strong_decay_backward(device):
             assert e < GRAD_TOL[name], (i, name, e)
 
 
+# float32 rows take the chunked float32 backward over the packed sequences (16-token chunks; its records are laid
+# out by (first row / 16) + sequence index): lengths around 16, empty sequences, one sequence per slot, many of them
+@pytest.mark.parametrize("lens,H", [([70, 128, 3, 190], 2), ([16, 0, 1, 17, 13, 0, 32], 3), ([200, 40], 40),
+                                    ([5] * 70, 1), ([15, 1] * 20, 2)])
+def test_varlen_float32_backward_matches_oracle_per_sequence(device, lens, H):
+    packed, parts, h0, cu = pack(lens, H, seed=7800 + H, dtype=torch.float32, tail=9)
+    T = packed[0].shape[1]
+    g = torch.Generator().manual_seed(H)
+    dO = torch.randn(1, T, H, 64, generator=g)
+    dS = 0.1 * torch.randn(len(lens), H, 64, 64, generator=g)
+    got = grads_packed(packed, h0, cu, dO, dS, device)
+    worst = 0.0
+    for i, (p, L) in enumerate(zip(parts, lens)):
+        if L == 0:
+            assert torch.equal(got[6][i].cpu(), dS[i]), i
+            continue
+        ref = orc.gradients(*p[:6], h0[i:i + 1], dO[:, cu[i]:cu[i + 1]], dS[i:i + 1])
+        for j, name in enumerate(GRAD_NAMES):
+            mine = got[j][i:i + 1] if name == "dh0" else got[j][:, cu[i]:cu[i + 1]]
+            assert mine.dtype == torch.float32
+            e = rel_l2(mine, ref[j])
+            worst = max(worst, e)
+            assert e < 1e-4, (i, L, name, e)
+    print(f"float32 lens={lens[:8]} H={H}: worst rel_l2 {worst:.2e}")
+    for j in range(6):
+        assert torch.count_nonzero(got[j][:, cu[-1]:]) == 0
+
+
+# the second case has more sequence-heads (1200) than the token-by-token kernel has workgroups (1024): some take two
+@pytest.mark.parametrize("lens,H,strong_seq", [([100, 64, 0, 30], 2, 1), ([7] * 299 + [20], 4, 299)])
+def test_varlen_float32_strong_decay_backward(device, lens, H, strong_seq):
+    """One sequence whose decays are too strong for the chunk form: the token-by-token kernel does the whole packed
+    call."""
+    packed, parts, h0, cu = pack(lens, H, seed=7900, dtype=torch.float32)
+    g = torch.Generator().manual_seed(2)
+    packed[1] = packed[1].clone()
+    packed[1][:, cu[strong_seq]:cu[strong_seq + 1]] = 2.0 + torch.randn(1, lens[strong_seq], H, 64, generator=g)
+    parts = [[x[:, cu[i]:cu[i + 1]] for x in packed] + [None] for i in range(len(lens))]
+    dO = torch.randn(1, cu[-1], H, 64, generator=g)
+    dS = 0.1 * torch.randn(len(lens), H, 64, 64, generator=g)
+    got = grads_packed(packed, h0, cu, dO, dS, device)
+    for i, (p, L) in enumerate(zip(parts, lens)):
+        if L == 0:
+            assert torch.equal(got[6][i].cpu(), dS[i]), i
+            continue
+        ref = orc.gradients(*p[:6], h0[i:i + 1], dO[:, cu[i]:cu[i + 1]], dS[i:i + 1])
+        for j, name in enumerate(GRAD_NAMES):
+            mine = got[j][i:i + 1] if name == "dh0" else got[j][:, cu[i]:cu[i + 1]]
+            assert torch.isfinite(mine).all()
+            assert rel_l2(mine, ref[j]) < 1e-4, (i, name)
+
+
 def test_varlen_bad_table_does_not_fault(device):
     """A table that lies (beyond T, decreasing) gives meaningless values but stays inside the tensors."""
     xs = make_inputs(1, 300, 2, 64, seed=7800, dtype=torch.bfloat16)
