@@ -273,6 +273,20 @@ int rwkv7_bwd_varlen(const void* r, const void* w, const void* k, const void* v,
                      void* dr, void* dw, void* dk, void* dv, void* da, void* db, float* dh0,
                      int T_total, int H, int K, int V, int dtype,
                      void* ws, size_t ws_bytes, void* stream);
+/* rwkv7_bwd_recurrent over packed sequences: the token-by-token float32 backward (bf16, f32 or f16 tensors,
+ * K = V = 64 or 128) with the arguments of rwkv7_bwd_varlen -- the gradients of packed rows at head size 128, which
+ * rwkv7_bwd_varlen does not take.  No counterpart in the reference, like the packed calls above.  Workspace: one
+ * state per segment of 64 tokens (32 at K = 128) for T_total / segment + n_seq segments per head, plus a segment's
+ * worth of states for each of at most 1024 (sequence, head) pairs walked at a time. */
+size_t rwkv7_bwd_recurrent_varlen_workspace_bytes(int n_seq, int T_total, int H, int K);
+int rwkv7_bwd_recurrent_varlen(const void* r, const void* w, const void* k, const void* v,
+                               const void* a, const void* b,
+                               const int32_t* cu_seqlens, int n_seq,
+                               const float* h0, int64_t h0_batch_stride,
+                               const void* d_o, const float* d_ht,
+                               void* dr, void* dw, void* dk, void* dv, void* da, void* db, float* dh0,
+                               int T_total, int H, int K, int V, int dtype,
+                               void* ws, size_t ws_bytes, void* stream);
 
 /* The float32 recurrent kernel for either dtype (inputs are widened on load):
  * the arithmetic of native_keras_op.py:85,87 one token at a time with the state

@@ -432,6 +432,36 @@ int rwkv7_bwd_varlen(const void* r, const void* w, const void* k, const void* v,
     return (int)rwkv7::launch_bwd_chunk(p, ws, static_cast<hipStream_t>(stream));
 }
 
+size_t rwkv7_bwd_recurrent_varlen_workspace_bytes(int n_seq, int T_total, int H, int K) {
+    if (n_seq < 1 || T_total < 1 || H < 1 || (K != 64 && K != 128)) return 0;
+    return rwkv7::bwd_recurrent_workspace_bytes(n_seq, T_total, H, K, true);
+}
+
+int rwkv7_bwd_recurrent_varlen(const void* r, const void* w, const void* k, const void* v, const void* a, const void* b,
+                               const int32_t* cu_seqlens, int n_seq, const float* h0, int64_t h0_batch_stride,
+                               const void* d_o, const float* d_ht,
+                               void* dr, void* dw, void* dk, void* dv, void* da, void* db, float* dh0,
+                               int T_total, int H, int K, int V, int dtype, void* ws, size_t ws_bytes, void* stream)
+{
+    int rc = check_seq(r, w, k, v, a, b, h0, h0_batch_stride, dr, nullptr, 1, T_total, H, K, V, dtype, true, true);
+    if (rc != RWKV7_OK) return rc;
+    rc = check_varlen(cu_seqlens, n_seq, T_total, H);
+    if (rc != RWKV7_OK) return rc;
+    if (!dw || !dk || !dv || !da || !db) return RWKV7_ERR_NULL_POINTER;
+    if (!aligned16(d_o) || !aligned16(d_ht) || !aligned16(dw) || !aligned16(dk) || !aligned16(dv) ||
+        !aligned16(da) || !aligned16(db) || !aligned16(dh0))
+        return RWKV7_ERR_ALIGNMENT;
+    const size_t need = rwkv7::bwd_recurrent_workspace_bytes(n_seq, T_total, H, K, true);
+    if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return RWKV7_ERR_WORKSPACE;
+    rwkv7::BwdArgs p;
+    p.r = r; p.w = w; p.k = k; p.v = v; p.a = a; p.b = b;
+    p.h0 = h0; p.h0_batch_stride = h0 ? h0_batch_stride : 0;
+    p.dO = d_o; p.dht = d_ht;
+    p.dr = dr; p.dw = dw; p.dk = dk; p.dv = dv; p.da = da; p.db = db; p.dh0 = dh0;
+    p.B = n_seq; p.T = T_total; p.H = H; p.dtype = dtype; p.cu = cu_seqlens;
+    return (int)rwkv7::launch_bwd_recurrent(p, K, ws, static_cast<hipStream_t>(stream));
+}
+
 /* ---- RWKV6 ------------------------------------------------------------------------------------- */
 namespace {
 int pack_rwkv6(const void* r, const void* k, const void* v, const void* w, const void* u,

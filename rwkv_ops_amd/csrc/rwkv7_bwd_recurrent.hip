@@ -61,11 +61,22 @@ template <int N> struct RecShape {
 
 int bwd_recurrent_segment(int N) { return N == 64 ? RecShape<64>::SEG : RecShape<128>::SEG; }
 
-size_t bwd_recurrent_workspace_bytes(int B, int T, int H, int N) {
+namespace {
+// packed sequences: (T_total / seg + n_seq) H records; scratch areas for at most WALK_MAX_GRID workgroups
+size_t rec_records(int B, int T, int H, int seg, bool varlen) {
+    return varlen ? ((size_t)(T / seg) + B) * H : (size_t)B * H * ((T + seg - 1) / seg);
+}
+size_t rec_areas(int B, int H, bool varlen) {
+    const size_t bh = (size_t)B * H;
+    return varlen && bh > (size_t)WALK_MAX_GRID ? (size_t)WALK_MAX_GRID : bh;
+}
+}  // namespace
+
+size_t bwd_recurrent_workspace_bytes(int B, int T, int H, int N, bool varlen) {
     const int seg = bwd_recurrent_segment(N);
     const size_t state = (size_t)N * N * 4;
-    const size_t nseg = (size_t)(T + seg - 1) / seg;
-    return (size_t)B * H * (nseg + seg) * state;             // stored segment states, then each workgroup's scratch
+    // stored segment states, then each workgroup's scratch
+    return (rec_records(B, T, H, seg, varlen) + rec_areas(B, H, varlen) * seg) * state;
 }
 
 template <typename T, int N>
@@ -77,14 +88,15 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
                           T* __restrict__ dr, T* __restrict__ dw, T* __restrict__ dk, T* __restrict__ dv,
                           T* __restrict__ da, T* __restrict__ db, float* __restrict__ dh0, int T_rows, int H,
                           int ckpt_per_head, int ckpt_step, const int* __restrict__ run_if_any, int n_flags,
-                          const int* __restrict__ cu, int n_bh)
+                          const int* __restrict__ cu, int n_bh, int cu_shift)
 {
     // ckpt: the state before token SEG * s is record ckpt_step * s of this head's ckpt_per_head records.
     // run_if_any (nullable): n_flags integers; the kernel runs only when one of them is not zero.
     // cu (nullable): packed sequences -- cumulative lengths of the n_bh / H sequences in one row of T_rows tokens;
-    // the checkpoints are then the records of the chunked float32 backward (sequence b, segment s: record
-    // ((first row / 16) + b + 4 s) H + h).  The grid may be smaller than n_bh: a workgroup takes every gridDim.x-th
-    // (sequence, head) and owns one scratch area.
+    // the checkpoints are then records of one per 2^cu_shift tokens laid out by slots (sequence b, segment s: record
+    // ((first row >> cu_shift) + b + s (SEG >> cu_shift)) H + h): cu_shift 4 for the records of the chunked float32
+    // backward, log2(SEG) for this backward's own forward pass.  The grid may be smaller than n_bh: a workgroup takes
+    // every gridDim.x-th (sequence, head) and owns one scratch area.
     constexpr int CPW = RecShape<N>::CPW, SEG = RecShape<N>::SEG;
     constexpr int VQ = CPW / 4;                  // lanes across a wave's columns, four columns each
     constexpr int ROWS = N / (64 / VQ);          // state rows per lane
@@ -126,9 +138,9 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
     }
     const int64_t base = (tok0 * H + hi) * N;
     const int nseg = (T_len + SEG - 1) / SEG;
-    const float* my_ckpt = cu != nullptr ? ckpt + (((tok0 >> 4) + bi) * H + hi) * (int64_t)(N * N)
+    const float* my_ckpt = cu != nullptr ? ckpt + (((tok0 >> cu_shift) + bi) * H + hi) * (int64_t)(N * N)
                                          : ckpt + (int64_t)bh * ckpt_per_head * (N * N);
-    const int64_t ckpt_stride = cu != nullptr ? (int64_t)4 * H * (N * N) : (int64_t)ckpt_step * (N * N);
+    const int64_t ckpt_stride = cu != nullptr ? (int64_t)(SEG >> cu_shift) * H * (N * N) : (int64_t)ckpt_step * (N * N);
 
     // one block of per-token vectors -> LDS as float (w as the decay d, and as dfac = dd/dw = -exp(w) d)
     auto stage_block = [&](int t0, int nt, bool reverse_pass) {
@@ -306,7 +318,7 @@ template <int N> constexpr size_t rec_lds_bytes() {
 template <typename T, int N>
 hipError_t launch_bwd_rec_t(const BwdArgs& p, const float* ckpt, float* scratch, hipStream_t stream,
                             int ckpt_per_head = 0, int ckpt_step = 1, const int* run_if_any = nullptr, int n_flags = 0,
-                            int max_grid = 0) {
+                            int max_grid = 0, int cu_shift = 4) {
     if (ckpt_per_head == 0) ckpt_per_head = (p.T + RecShape<N>::SEG - 1) / RecShape<N>::SEG;
     const int n_bh = p.B * p.H;
     const int grid = max_grid > 0 && n_bh > max_grid ? max_grid : n_bh;
@@ -317,7 +329,7 @@ hipError_t launch_bwd_rec_t(const BwdArgs& p, const float* ckpt, float* scratch,
     bwd_recurrent_kernel<T, N><<<dim3((unsigned)grid), dim3(256), lds, stream>>>(
         (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, (const T*)p.a, (const T*)p.b,
         (const T*)p.dO, p.dht, ckpt, scratch, (T*)p.dr, (T*)p.dw, (T*)p.dk, (T*)p.dv, (T*)p.da, (T*)p.db,
-        p.dh0, p.T, p.H, ckpt_per_head, ckpt_step, run_if_any, n_flags, p.cu, n_bh);
+        p.dh0, p.T, p.H, ckpt_per_head, ckpt_step, run_if_any, n_flags, p.cu, n_bh, cu_shift);
     return hipGetLastError();
 }
 }  // namespace
@@ -333,25 +345,35 @@ hipError_t launch_bwd_recurrent_walk_f32(const BwdArgs& p, const float* states16
 
 hipError_t launch_bwd_recurrent(const BwdArgs& p, int N, void* ws, hipStream_t stream) {
     const int seg = bwd_recurrent_segment(N);
-    const size_t nseg = (size_t)(p.T + seg - 1) / seg;
+    const bool varlen = p.cu != nullptr;
     float* ckpt = static_cast<float*>(ws);
-    float* scratch = ckpt + (size_t)p.B * p.H * nseg * N * N;
+    float* scratch = ckpt + rec_records(p.B, p.T, p.H, seg, varlen) * N * N;
     // launch 1: the forward once more, leaving the state at the start of every segment
     SeqArgs f{};
     f.r = p.r; f.w = p.w; f.k = p.k; f.v = p.v; f.a = p.a; f.b = p.b;
     f.h0 = p.h0; f.h0_batch_stride = p.h0 ? p.h0_batch_stride : 0;
-    f.B = p.B; f.T = p.T; f.H = p.H; f.N = N; f.dtype = p.dtype;
-    // (float32 tensors at head size 64 beyond a dozen tokens: the chunked float32 forward, otherwise the recurrent one)
-    hipError_t e = (N == 64 && p.dtype == RWKV7_DTYPE_F32 && p.T > 12) ? launch_fwd_chunk_f32_states(f, ckpt, seg, stream)
-                                                                      : launch_fwd_recurrent_states(f, ckpt, seg, stream);
+    f.B = p.B; f.T = p.T; f.H = p.H; f.N = N; f.dtype = p.dtype; f.cu = p.cu;
+    hipError_t e;
+    if (varlen) {                      // rows of the gradients behind the last sequence
+        TailFill tail;
+        tail.p[0] = p.dr; tail.p[1] = p.dw; tail.p[2] = p.dk; tail.p[3] = p.dv; tail.p[4] = p.da; tail.p[5] = p.db;
+        tail.n = 6; tail.row_bytes = (int64_t)p.H * N * (p.dtype == RWKV7_DTYPE_F32 ? 4 : 2);
+        e = launch_chunk_items(seq_layout(f, nullptr), nullptr, nullptr, 0, nullptr, tail, stream);
+        if (e != hipSuccess) return e;
+    }
+    // (dense float32 tensors at head size 64 beyond a dozen tokens: the chunked float32 forward, otherwise the recurrent one)
+    e = (!varlen && N == 64 && p.dtype == RWKV7_DTYPE_F32 && p.T > 12) ? launch_fwd_chunk_f32_states(f, ckpt, seg, stream)
+                                                                       : launch_fwd_recurrent_states(f, ckpt, seg, stream);
     if (e != hipSuccess) return e;
+    // packed: the records lie by slots of one per segment, and at most WALK_MAX_GRID workgroups walk
+    const int grid = varlen ? WALK_MAX_GRID : 0, shift = seg == 64 ? 6 : 5;
     if (N == 128)
-        return p.dtype == RWKV7_DTYPE_BF16  ? launch_bwd_rec_t<bf16_t, 128>(p, ckpt, scratch, stream)
-               : p.dtype == RWKV7_DTYPE_F16 ? launch_bwd_rec_t<f16_t, 128>(p, ckpt, scratch, stream)
-                                            : launch_bwd_rec_t<float, 128>(p, ckpt, scratch, stream);
-    return p.dtype == RWKV7_DTYPE_BF16  ? launch_bwd_rec_t<bf16_t, 64>(p, ckpt, scratch, stream)
-           : p.dtype == RWKV7_DTYPE_F16 ? launch_bwd_rec_t<f16_t, 64>(p, ckpt, scratch, stream)
-                                        : launch_bwd_rec_t<float, 64>(p, ckpt, scratch, stream);
+        return p.dtype == RWKV7_DTYPE_BF16  ? launch_bwd_rec_t<bf16_t, 128>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)
+               : p.dtype == RWKV7_DTYPE_F16 ? launch_bwd_rec_t<f16_t, 128>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)
+                                            : launch_bwd_rec_t<float, 128>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift);
+    return p.dtype == RWKV7_DTYPE_BF16  ? launch_bwd_rec_t<bf16_t, 64>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)
+           : p.dtype == RWKV7_DTYPE_F16 ? launch_bwd_rec_t<f16_t, 64>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)
+                                        : launch_bwd_rec_t<float, 64>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift);
 }
 
 }  // namespace rwkv7

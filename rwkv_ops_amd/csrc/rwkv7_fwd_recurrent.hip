@@ -42,8 +42,10 @@ void fwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
                           T* __restrict__ o, float* __restrict__ ht, SeqLayout L,
                           float* __restrict__ seg_states = nullptr, int seg = 0)
 {
-    // seg_states (dense batches only): the state BEFORE token t is stored for every t that is a multiple of `seg`
-    // (a multiple of REC_TB), [workgroup][t / seg][N][N]: what the recurrent backward restarts from.  o may then be NULL.
+    // seg_states: the state BEFORE token t is stored for every t that is a multiple of `seg` (a multiple of REC_TB):
+    // what the recurrent backward restarts from; o may then be NULL.  Dense batches: [workgroup][t / seg][N][N].
+    // Packed sequences: sequence b owns the slots from (first row / seg) + b on (at most len / seg + 1 of them, never
+    // the next sequence's), record (slot + t / seg) H + h; (T_total / seg + n_seq) H records in all.
     constexpr int VQ = CPW / 4;                  // lanes across a wave's columns, four columns each
     constexpr int ROWS = N / (64 / VQ);          // state rows per lane
     constexpr int NT = 64 * (N / CPW);           // threads
@@ -132,7 +134,9 @@ void fwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
         request(t0 + REC_TB);
         if (seg_states != nullptr && t0 % seg == 0) {
             const int nseg = (T_len + seg - 1) / seg;
-            float* dst = seg_states + ((int64_t)blockIdx.x * nseg + t0 / seg) * (N * N) + tile;
+            const int64_t rec = L.cu != nullptr ? (sp.tok0 / seg + bi + t0 / seg) * H + hi
+                                                : (int64_t)blockIdx.x * nseg + t0 / seg;
+            float* dst = seg_states + rec * (N * N) + tile;
 #pragma unroll
             for (int i = 0; i < ROWS; ++i) *reinterpret_cast<float4_t*>(dst + i * N) = s[i];
         }
@@ -201,7 +205,8 @@ static hipError_t launch_states_t(const SeqArgs& p, float* states, int seg, hipS
     return hipGetLastError();
 }
 
-// the forward without outputs, storing the state at the start of every segment of `seg` tokens (dense batches)
+// the forward without outputs, storing the state at the start of every segment of `seg` tokens (dense batches, or
+// packed sequences, p.cu: see the kernel for where the records go)
 hipError_t launch_fwd_recurrent_states(const SeqArgs& p, float* states, int seg, hipStream_t stream) {
     if (p.N == 128)
         return p.dtype == RWKV7_DTYPE_BF16  ? launch_states_t<bf16_t, 128>(p, states, seg, stream)

@@ -83,9 +83,9 @@ hipError_t launch_chunk_items(const SeqLayout& L, void* items, const float* src,
 // chunked bf16 backward; ws must hold bwd_chunk_workspace_bytes(B, T, H) bytes, 256-byte aligned
 size_t bwd_chunk_workspace_bytes(int B, int T, int H, bool varlen = false);
 hipError_t launch_bwd_chunk(const BwdArgs& p, void* ws, hipStream_t stream);
-// float32 recurrent backward for any dtype, K = V = N in {64, 128}, dense batches (p.cu == NULL):
+// float32 recurrent backward for any dtype, K = V = N in {64, 128}, dense batches or packed sequences (p.cu):
 // ws holds bwd_recurrent_workspace_bytes(B, T, H, N) bytes (segment states, then per-workgroup scratch)
-size_t bwd_recurrent_workspace_bytes(int B, int T, int H, int N);
+size_t bwd_recurrent_workspace_bytes(int B, int T, int H, int N, bool varlen = false);
 hipError_t launch_bwd_recurrent(const BwdArgs& p, int N, void* ws, hipStream_t stream);
 hipError_t launch_fwd_recurrent_states(const SeqArgs& p, float* states, int seg, hipStream_t stream);
 // its second launch alone, float32 tensors at K = V = 64, over states stored every 16 tokens; runs only when one of

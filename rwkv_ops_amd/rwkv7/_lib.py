@@ -41,6 +41,8 @@ SIGNATURES = {
     "rwkv7_fwd_varlen": (_I, [_P] * 6 + [_P, _I, _P, _I64, _P, _P] + [_I] * 5 + [_P, _SZ, _P]),
     "rwkv7_bwd_varlen_workspace_bytes": (_SZ, [_I, _I, _I, _I]),
     "rwkv7_bwd_varlen": (_I, [_P] * 6 + [_P, _I, _P, _I64, _P, _P] + [_P] * 7 + [_I] * 5 + [_P, _SZ, _P]),
+    "rwkv7_bwd_recurrent_varlen_workspace_bytes": (_SZ, [_I, _I, _I, _I]),
+    "rwkv7_bwd_recurrent_varlen": (_I, [_P] * 6 + [_P, _I, _P, _I64, _P, _P] + [_P] * 7 + [_I] * 5 + [_P, _SZ, _P]),
     "rwkv6_fwd_workspace_bytes": (_SZ, [_I, _I, _I, _I]),
     "rwkv6_fwd": (_I, [_P] * 5 + [_P, _I, _P, _P, _P] + [_I] * 6 + [_P, _SZ, _P]),
     "rwkv6_bwd_workspace_bytes": (_SZ, [_I, _I, _I, _I]),

@@ -316,6 +316,37 @@ def _(r, w, k, v, a, b, h0, d_o, d_ht, cu):
         r.new_empty((cu.numel() - 1, H, N, N), dtype=torch.float32),)
 
 
+@torch.library.custom_op("rwkv_ops_amd::rwkv7_bwd_recurrent_varlen", mutates_args=(), device_types="cuda")
+def rwkv7_bwd_recurrent_varlen(r: torch.Tensor, w: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                               a: torch.Tensor, b: torch.Tensor, h0: Optional[torch.Tensor],
+                               d_o: Optional[torch.Tensor], d_ht: Optional[torch.Tensor], cu: torch.Tensor
+                               ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor,
+                                          torch.Tensor, torch.Tensor]:
+    """Gradients of ``rwkv7_fwd_varlen`` from the float32 recurrent backward: any of the three dtypes, head size 64
+    or 128 (what packed rows at head size 128 get); same arguments and results as ``rwkv7_bwd_varlen``."""
+    lib = _lib.load()
+    _, T, H, N = r.shape
+    n_seq = cu.numel() - 1
+    grads = [torch.empty_like(r) for _ in range(6)]
+    dh0 = torch.empty((n_seq, H, N, N), dtype=torch.float32, device=r.device)
+    with _on_device(r.device):
+        ws_bytes = lib.rwkv7_bwd_recurrent_varlen_workspace_bytes(n_seq, T, H, N)
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=r.device)
+        rc = lib.rwkv7_bwd_recurrent_varlen(_ptr(r), _ptr(w), _ptr(k), _ptr(v), _ptr(a), _ptr(b), _ptr(cu), n_seq,
+                                            _ptr(h0), _h0_stride(h0, n_seq, H), _ptr(d_o), _ptr(d_ht),
+                                            *[_ptr(x) for x in grads], _ptr(dh0),
+                                            T, H, N, N, _dtype_code(r.dtype), _ptr(ws), ws_bytes, _stream_ptr(r.device))
+    _lib.check(rc, "rwkv7_bwd_recurrent_varlen")
+    return (*grads, dh0)
+
+
+@rwkv7_bwd_recurrent_varlen.register_fake
+def _(r, w, k, v, a, b, h0, d_o, d_ht, cu):
+    _, T, H, N = r.shape
+    return tuple(torch.empty_like(r) for _ in range(6)) + (
+        r.new_empty((cu.numel() - 1, H, N, N), dtype=torch.float32),)
+
+
 def _fwd_varlen_setup_context(ctx, inputs, output):
     r, w, k, v, a, b, h0, want_state, cu = inputs
     ctx.save_for_backward(r, w, k, v, a, b, h0, cu)
@@ -327,12 +358,19 @@ def _fwd_varlen_backward(ctx, d_o, d_ht):
     dt = r.dtype
     # float32 rows at head size 64 keep float32 (the chunked float32 backward); float16 rows are rounded to bf16 as in
     # the dense call
-    exact = dt == torch.bfloat16 or (dt == torch.float32 and r.shape[-1] == HEAD_SIZE)
-    cast = (lambda t: t) if exact else (lambda t: t.to(torch.bfloat16))
-    d_o_c = None if d_o is None else cast(d_o.to(dt)).contiguous()
     d_ht_c = None
     if ctx.want_state and d_ht is not None and d_ht.numel() > 0:
         d_ht_c = d_ht.to(torch.float32).contiguous()
+    if r.shape[-1] != HEAD_SIZE:
+        # head size 128 has no chunked backward: the float32 recurrent backward, which reads any of the three dtypes
+        d_o_c = None if d_o is None else d_o.to(dt).contiguous()
+        dr, dw, dk, dv, da, db, dh0 = torch.ops.rwkv_ops_amd.rwkv7_bwd_recurrent_varlen(
+            r, w, k, v, a, b, h0, d_o_c, d_ht_c, cu)
+        g0 = dh0 if (h0 is not None and ctx.needs_input_grad[6]) else None
+        return dr, dw, dk, dv, da, db, g0, None, None
+    exact = dt == torch.bfloat16 or dt == torch.float32
+    cast = (lambda t: t) if exact else (lambda t: t.to(torch.bfloat16))
+    d_o_c = None if d_o is None else cast(d_o.to(dt)).contiguous()
     dr, dw, dk, dv, da, db, dh0 = torch.ops.rwkv_ops_amd.rwkv7_bwd_varlen(
         cast(r), cast(w), cast(k), cast(v), cast(a), cast(b), h0, d_o_c, d_ht_c, cu)
     g0 = dh0 if (h0 is not None and ctx.needs_input_grad[6]) else None
@@ -490,11 +528,6 @@ def _as_cu_seqlens(cu_seqlens, T: int, device: torch.device) -> torch.Tensor:
     return cu_seqlens.to(device=device, dtype=torch.int32).contiguous()
 
 
-def _no_wide_gradients(*tensors) -> None:
-    if tensors[0].shape[-1] != HEAD_SIZE and not _direct(*tensors) and not torch.compiler.is_compiling():
-        raise NotImplementedError(f"head size {tensors[0].shape[-1]} with cu_seqlens: only the forward is built "
-                                  f"(packed-sequence gradients need K = V = {HEAD_SIZE}); call under torch.no_grad()")
-
 
 def _check_inputs(r, w, k, v, a, b, initial_state, head_first, mapped=False):
     for name, x in zip("rwkvab", (r, w, k, v, a, b)):
@@ -603,7 +636,6 @@ def _generalized_delta_rule_varlen(r, w, k, v, a, b, initial_state, output_final
     r_, w_, k_, v_, a_, b_ = (_prepare(x, dt, False) for x in (r, w, k, v, a, b))
     cu = _as_cu_seqlens(cu_seqlens, r_.shape[1], r_.device)
     h0 = None if initial_state is None else initial_state.to(torch.float32).contiguous()
-    _no_wide_gradients(r_, w_, k_, v_, a_, b_, h0)
     if _direct(r_, w_, k_, v_, a_, b_, h0):
         out, state = _fwd_varlen_impl(r_, w_, k_, v_, a_, b_, h0, bool(output_final_state), cu)
     else:

@@ -7,6 +7,8 @@ bf16 backward on the same inputs, whose own error is the larger one."""
 import pytest
 import torch
 
+import rwkv_ops_amd  # noqa: F401  (registers the torch.library ops)
+
 from oracle import rwkv7_native as orc
 from rwkv_ops_amd.rwkv7 import _lib
 from rwkv_ops_amd.synthetic import GRAD_NAMES, GRAD_TOL, make_inputs, rel_l2
@@ -105,6 +107,38 @@ def test_rwkv7_bwd_routes_short_float32_calls_to_the_recurrent_backward(device):
             assert torch.equal(x, y) if same else rel_l2(x, y) < 1e-5
         if same:
             assert lib.rwkv7_bwd_workspace_bytes(B, T, H, _lib.DTYPE_F32) == lib.rwkv7_bwd_recurrent_workspace_bytes(B, T, H, 64)
+
+
+def test_recurrent_backward_over_packed_sequences(device):
+    """rwkv7_bwd_recurrent_varlen at head size 64 (segments of 64 tokens, their records by (first row / 64) + sequence
+    index) against the chunked float32 backward over the same packed float32 rows, and sequence by sequence against
+    the dense recurrent call (whose segment states come from the chunked float32 forward, the packed call's from the
+    recurrent one: equal to rounding)."""
+    lens, H, N = [130, 0, 64, 1, 65, 7], 2, 64
+    parts = [make_inputs(1, max(L, 1), H, N, seed=3400 + i, dtype=torch.float32) for i, L in enumerate(lens)]
+    parts = [[x[:, :L] for x in p[:6]] + [p[6]] for p, L in zip(parts, lens)]
+    packed = [torch.cat([p[j] for p in parts], dim=1).contiguous().to(device) for j in range(6)]
+    h0 = torch.cat([p[6] for p in parts], dim=0).contiguous().to(device)
+    cu = [0]
+    for L in lens:
+        cu.append(cu[-1] + L)
+    cu_d = torch.tensor(cu, dtype=torch.int32, device=device)
+    g = torch.Generator().manual_seed(6)
+    dO = torch.randn(1, cu[-1], H, N, generator=g).to(device)
+    dS = (0.1 * torch.randn(len(lens), H, N, N, generator=g)).to(device)
+    rec = torch.ops.rwkv_ops_amd.rwkv7_bwd_recurrent_varlen(*packed, h0, dO, dS, cu_d)
+    chk = torch.ops.rwkv_ops_amd.rwkv7_bwd_varlen(*packed, h0, dO, dS, cu_d)
+    for n, x, y in zip(GRAD_NAMES, rec, chk):
+        assert rel_l2(x, y) < 1e-5, n
+    for i, L in enumerate(lens):
+        if L == 0:
+            assert torch.equal(rec[6][i], dS[i])
+            continue
+        one = torch.ops.rwkv_ops_amd.rwkv7_bwd_recurrent(*[x[:, cu[i]:cu[i + 1]].contiguous() for x in packed],
+                                                         h0[i:i + 1], dO[:, cu[i]:cu[i + 1]].contiguous(), dS[i:i + 1])
+        for j, n in enumerate(GRAD_NAMES):
+            mine = rec[j][i:i + 1] if n == "dh0" else rec[j][:, cu[i]:cu[i + 1]]
+            assert rel_l2(mine, one[j]) < 2e-6, (i, n)
 
 
 def test_recurrent_and_chunked_backward_agree(device):
