@@ -52,10 +52,15 @@ __device__ __forceinline__ float reduce_cols(float x) {
 
 __device__ __forceinline__ float dot4(float4_t a, float4_t b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
 
-template <int N> struct RecShape {
-    static constexpr int CPW = N == 64 ? 16 : 32;            // value columns per wave
+template <int N, int VS = 1> struct RecShape {
+    static constexpr int CPW = (N == 64 ? 16 : 32) / VS;     // value columns per wave (four waves cover N / VS columns)
     static constexpr int SEG = N == 64 ? 64 : 32;            // tokens per segment
 };
+// Head size 128 with few (batch, head) pairs: the value columns of a head go to VS = 2 workgroups (the walk is bound by
+// the vector throughput of a CU, and half of the CUs would have no head); each leaves its partial sums of the five
+// [token][key] gradients in the workspace and a small kernel adds them.
+constexpr int VSPLIT_MAX_BH = 192;
+bool splits_values(int B, int H, int N, bool varlen) { return N == 128 && !varlen && (int64_t)B * H <= VSPLIT_MAX_BH; }
 
 }  // namespace
 
@@ -75,11 +80,14 @@ size_t rec_areas(int B, int H, bool varlen) {
 size_t bwd_recurrent_workspace_bytes(int B, int T, int H, int N, bool varlen) {
     const int seg = bwd_recurrent_segment(N);
     const size_t state = (size_t)N * N * 4;
-    // stored segment states, then each workgroup's scratch
-    return (rec_records(B, T, H, seg, varlen) + rec_areas(B, H, varlen) * seg) * state;
+    const bool split = splits_values(B, H, N, varlen);
+    // stored segment states, then each workgroup's scratch, then (value columns split over two workgroups) the two
+    // parts' sums of the five [token][key] gradients
+    return (rec_records(B, T, H, seg, varlen) + rec_areas(B, H, varlen) * (split ? 2 : 1) * seg) * state +
+           (split ? (size_t)2 * 5 * B * T * H * N * 4 : 0);
 }
 
-template <typename T, int N>
+template <typename T, int N, int VS = 1>
 __global__ __launch_bounds__(256)
 void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, const T* __restrict__ k,
                           const T* __restrict__ v, const T* __restrict__ a, const T* __restrict__ b,
@@ -88,8 +96,10 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
                           T* __restrict__ dr, T* __restrict__ dw, T* __restrict__ dk, T* __restrict__ dv,
                           T* __restrict__ da, T* __restrict__ db, float* __restrict__ dh0, int T_rows, int H,
                           int ckpt_per_head, int ckpt_step, const int* __restrict__ run_if_any, int n_flags,
-                          const int* __restrict__ cu, int n_bh, int cu_shift)
+                          const int* __restrict__ cu, int n_bh, int cu_shift, float* __restrict__ pbuf)
 {
+    // VS > 1 (dense batches): workgroup item = (batch, head) * VS + part owns the value columns (N / VS) * part .. of
+    // its head and writes its sums over them of dr, dk, db, dw, da to pbuf [VS][5][B * T_rows][H][N] (float32).
     // ckpt: the state before token SEG * s is record ckpt_step * s of this head's ckpt_per_head records.
     // run_if_any (nullable): n_flags integers; the kernel runs only when one of them is not zero.
     // cu (nullable): packed sequences -- cumulative lengths of the n_bh / H sequences in one row of T_rows tokens;
@@ -97,11 +107,11 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
     // ((first row >> cu_shift) + b + s (SEG >> cu_shift)) H + h): cu_shift 4 for the records of the chunked float32
     // backward, log2(SEG) for this backward's own forward pass.  The grid may be smaller than n_bh: a workgroup takes
     // every gridDim.x-th (sequence, head) and owns one scratch area.
-    constexpr int CPW = RecShape<N>::CPW, SEG = RecShape<N>::SEG;
+    constexpr int CPW = RecShape<N, VS>::CPW, SEG = RecShape<N, VS>::SEG;
     constexpr int VQ = CPW / 4;                  // lanes across a wave's columns, four columns each
     constexpr int ROWS = N / (64 / VQ);          // state rows per lane
-    constexpr int PARTS = N / CPW;               // waves
-    static_assert(PARTS == 4, "four waves per (batch, head)");
+    constexpr int PARTS = N / VS / CPW;          // waves
+    static_assert(PARTS == 4, "four waves per workgroup");
     // staged per-token vectors of one block, as float: a, d, b, k, v (both passes), r, do, dfac (reverse pass)
     enum { Q_A = 0, Q_D, Q_B, Q_K, Q_V, Q_R, Q_DO, Q_DF, Q_COUNT };
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -121,12 +131,13 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
     const int lane = tid & 63;
     const int wave = tid >> 6;                   // which CPW value columns
     const int ks = lane / VQ, vq = lane % VQ;
-    const int col0 = CPW * wave + 4 * vq;        // this lane's four value columns
     const int row0 = ROWS * ks;                  // this lane's first state row
-    const int tile = row0 * N + col0;
     const int64_t step = (int64_t)H * N;
     float* my_scr = scratch + (int64_t)blockIdx.x * SEG * (N * N);
-  for (int bh = blockIdx.x; bh < n_bh; bh += gridDim.x) {
+  for (int item = blockIdx.x; item < n_bh * VS; item += gridDim.x) {
+    const int bh = item / VS, vs = item % VS;
+    const int col0 = (N / VS) * vs + CPW * wave + 4 * vq;    // this lane's four value columns
+    const int tile = row0 * N + col0;
     const int hi = bh % H, bi = bh / H;
     int64_t tok0 = (int64_t)bi * T_rows;
     int T_len = T_rows;
@@ -295,8 +306,13 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
 #pragma unroll
                     for (int p = 0; p < PARTS; ++p) sum += *reinterpret_cast<const float4_t*>(&part[q][tt][p][e0]);
                     if (q == O_DD) sum = sum * *reinterpret_cast<const float4_t*>(&stage[Q_DF][tt][e0]);
-                    const float o4[4] = {sum.x, sum.y, sum.z, sum.w};
-                    Io<T>::store4(outs[q] + off, o4);
+                    if constexpr (VS > 1) {
+                        const int64_t all = (int64_t)(n_bh / H) * T_rows * step;       // elements of one tensor
+                        *reinterpret_cast<float4_t*>(pbuf + ((int64_t)vs * O_COUNT + q) * all + off) = sum;
+                    } else {
+                        const float o4[4] = {sum.x, sum.y, sum.z, sum.w};
+                        Io<T>::store4(outs[q] + off, o4);
+                    }
                 }
             }
         }
@@ -310,26 +326,50 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
   }
 }
 
+// out[q] = sum over the VS parts of pbuf [VS][5][elements], four elements per thread
+template <typename T, int VS>
+__global__ __launch_bounds__(256)
+void bwd_recurrent_combine_kernel(const float* __restrict__ pbuf, T* __restrict__ dr, T* __restrict__ dk,
+                                  T* __restrict__ db, T* __restrict__ dw, T* __restrict__ da, int64_t elements)
+{
+    const int64_t i4 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i4 >= elements) return;
+    T* const outs[5] = {dr, dk, db, dw, da};      // the order of O_DR .. O_DA
+#pragma unroll
+    for (int q = 0; q < 5; ++q) {
+        float4_t sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int p = 0; p < VS; ++p) sum += *reinterpret_cast<const float4_t*>(pbuf + ((int64_t)p * 5 + q) * elements + i4);
+        const float o4[4] = {sum.x, sum.y, sum.z, sum.w};
+        Io<T>::store4(outs[q] + i4, o4);
+    }
+}
+
 namespace {
 template <int N> constexpr size_t rec_lds_bytes() {
     return sizeof(float) * ((size_t)8 * RB_TB * N + (size_t)RecShape<N>::SEG * N + (size_t)5 * RB_TB * 4 * N);
 }
 
-template <typename T, int N>
+template <typename T, int N, int VS = 1>
 hipError_t launch_bwd_rec_t(const BwdArgs& p, const float* ckpt, float* scratch, hipStream_t stream,
                             int ckpt_per_head = 0, int ckpt_step = 1, const int* run_if_any = nullptr, int n_flags = 0,
-                            int max_grid = 0, int cu_shift = 4) {
+                            int max_grid = 0, int cu_shift = 4, float* pbuf = nullptr) {
     if (ckpt_per_head == 0) ckpt_per_head = (p.T + RecShape<N>::SEG - 1) / RecShape<N>::SEG;
     const int n_bh = p.B * p.H;
-    const int grid = max_grid > 0 && n_bh > max_grid ? max_grid : n_bh;
+    const int grid = max_grid > 0 && n_bh > max_grid ? max_grid : n_bh * VS;
     constexpr size_t lds = rec_lds_bytes<N>();
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_recurrent_kernel<T, N>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_recurrent_kernel<T, N, VS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
-    bwd_recurrent_kernel<T, N><<<dim3((unsigned)grid), dim3(256), lds, stream>>>(
+    bwd_recurrent_kernel<T, N, VS><<<dim3((unsigned)grid), dim3(256), lds, stream>>>(
         (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, (const T*)p.a, (const T*)p.b,
         (const T*)p.dO, p.dht, ckpt, scratch, (T*)p.dr, (T*)p.dw, (T*)p.dk, (T*)p.dv, (T*)p.da, (T*)p.db,
-        p.dh0, p.T, p.H, ckpt_per_head, ckpt_step, run_if_any, n_flags, p.cu, n_bh, cu_shift);
+        p.dh0, p.T, p.H, ckpt_per_head, ckpt_step, run_if_any, n_flags, p.cu, n_bh, cu_shift, pbuf);
+    e = hipGetLastError();
+    if (e != hipSuccess || VS == 1) return e;
+    const int64_t elements = (int64_t)p.B * p.T * p.H * N;
+    bwd_recurrent_combine_kernel<T, VS><<<dim3((unsigned)((elements / 4 + 255) / 256)), dim3(256), 0, stream>>>(
+        pbuf, (T*)p.dr, (T*)p.dk, (T*)p.db, (T*)p.dw, (T*)p.da, elements);
     return hipGetLastError();
 }
 }  // namespace
@@ -367,6 +407,12 @@ hipError_t launch_bwd_recurrent(const BwdArgs& p, int N, void* ws, hipStream_t s
     if (e != hipSuccess) return e;
     // packed: the records lie by slots of one per segment, and at most WALK_MAX_GRID workgroups walk
     const int grid = varlen ? WALK_MAX_GRID : 0, shift = seg == 64 ? 6 : 5;
+    if (splits_values(p.B, p.H, N, varlen)) {
+        float* pbuf = scratch + (size_t)p.B * p.H * 2 * seg * N * N;
+        return p.dtype == RWKV7_DTYPE_BF16  ? launch_bwd_rec_t<bf16_t, 128, 2>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, 0, shift, pbuf)
+               : p.dtype == RWKV7_DTYPE_F16 ? launch_bwd_rec_t<f16_t, 128, 2>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, 0, shift, pbuf)
+                                            : launch_bwd_rec_t<float, 128, 2>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, 0, shift, pbuf);
+    }
     if (N == 128)
         return p.dtype == RWKV7_DTYPE_BF16  ? launch_bwd_rec_t<bf16_t, 128>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)
                : p.dtype == RWKV7_DTYPE_F16 ? launch_bwd_rec_t<f16_t, 128>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)

@@ -194,3 +194,26 @@ def test_packed_gradients(device, dtype, tol):
             assert e < (1e-4 if name == "dh0" else (tol if L * H * N >= 4096 else 2 * tol)), (i, L, name, e)
     for j in range(6):
         assert got[j].dtype == dtype and torch.count_nonzero(got[j][:, cu[-1]:]) == 0
+
+
+def test_gradients_with_many_heads(device):
+    """At most 192 (batch, head) pairs: the value columns of a head are split over two workgroups, whose partial sums
+    a second kernel adds (the shapes above); beyond: one workgroup per pair.  Here 208 pairs, and the same tensors'
+    first 3 batch rows (24 pairs) through the split form: both against float32 autograd through the oracle, and
+    against each other (different orders of the same float32 sums)."""
+    B, T, H = 26, 20, 8
+    xs = make_inputs(B, T, H, N, seed=9500, dtype=torch.float32)
+    g = torch.Generator().manual_seed(9501)
+    dO = torch.randn(B, T, H, N, generator=g)
+    dS = 0.1 * torch.randn(B, H, N, N, generator=g)
+    ref = orc.gradients(*xs[:6], xs[6], dO, dS)
+    got = {}
+    for rows in (B, 3):
+        leaves = [x[:rows].contiguous().to(device).requires_grad_(True) for x in xs]
+        o, s = rwkv_ops_amd.generalized_delta_rule(*leaves[:6], initial_state=leaves[6])
+        loss = (o * dO[:rows].to(device)).sum() + (s * dS[:rows].to(device)).sum()
+        got[rows] = torch.autograd.grad(loss, leaves)
+        for name, g_, r_ in zip(["dr", "dw", "dk", "dv", "da", "db", "dh0"], got[rows], ref):
+            assert rel_l2(g_, r_[:rows]) < 1e-4, (rows, name)
+    for a_, b_ in zip(got[B], got[3]):
+        assert rel_l2(a_[:3], b_) < 2e-6
