@@ -23,6 +23,7 @@
 // kernel's cross-lane reduction inside the wave; sums over V (dr, dk, db, dd, da) cross the waves, but nothing
 // later depends on them, so each wave leaves its partial sums in LDS and the workgroup adds them up and writes
 // the five output rows once per block of RB_TB tokens.
+#include <type_traits>
 #include "rwkv7_common.h"
 #include "rwkv7_kernels.h"
 #include "../../include/rwkv7_mi355x.h"
@@ -31,11 +32,12 @@ namespace rwkv7 {
 
 namespace {
 
-constexpr int RB_TB = 8;                         // tokens per staged block
 
 template <int VQ>
 __device__ __forceinline__ float reduce_rows(float x) {      // sum over the lanes that share lane % VQ
-    if constexpr (VQ == 4)
+    if constexpr (VQ == 2)
+        x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x122, 0xf, 0xf, true));   // row_ror:2
+    if constexpr (VQ <= 4)
         x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x124, 0xf, 0xf, true));   // row_ror:4
     return sum_lane_groups_of_8(x);
 }
@@ -44,7 +46,8 @@ __device__ __forceinline__ float reduce_rows(float x) {      // sum over the lan
 template <int VQ>
 __device__ __forceinline__ float reduce_cols(float x) {
     x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x101, 0xf, 0xf, true));       // row_shl:1
-    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x102, 0xf, 0xf, true));       // row_shl:2
+    if constexpr (VQ >= 4)
+        x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x102, 0xf, 0xf, true));   // row_shl:2
     if constexpr (VQ == 8)
         x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x104, 0xf, 0xf, true));   // row_shl:4
     return x;
@@ -52,14 +55,20 @@ __device__ __forceinline__ float reduce_cols(float x) {
 
 __device__ __forceinline__ float dot4(float4_t a, float4_t b) { return a.x * b.x + a.y * b.y + a.z * b.z + a.w * b.w; }
 
-template <int N, int VS = 1> struct RecShape {
-    static constexpr int CPW = (N == 64 ? 16 : 32) / VS;     // value columns per wave (four waves cover N / VS columns)
+template <int N, int VS = 1, int W = 4> struct RecShape {
+    static constexpr int CPW = N / VS / W;                   // value columns per wave (W waves cover N / VS columns)
     static constexpr int SEG = N == 64 ? 64 : 32;            // tokens per segment
+    static constexpr int RB = W * N > 512 ? 4 : 8;           // tokens per staged block (the partial sums fill 80 KiB of LDS)
+    // The walk back keeps the state before every KEEP-th token of a segment and takes the others by steps forward
+    // from it (three multiply-adds per element and no sum across lanes): a quarter of the scratch traffic, which
+    // is what bounds the walk when there are more heads than CUs.
+    static constexpr int KEEP = 4;
 };
 // Head size 128 with few (batch, head) pairs: the value columns of a head go to VS = 2 workgroups (the walk is bound by
 // the vector throughput of a CU, and half of the CUs would have no head); each leaves its partial sums of the five
 // [token][key] gradients in the workspace and a small kernel adds them.
 constexpr int VSPLIT_MAX_BH = 192;
+constexpr int W_SPLIT = 8, W_128 = 8, W_64 = 4;           // waves per workgroup
 bool splits_values(int B, int H, int N, bool varlen) { return N == 128 && !varlen && (int64_t)B * H <= VSPLIT_MAX_BH; }
 
 }  // namespace
@@ -83,12 +92,12 @@ size_t bwd_recurrent_workspace_bytes(int B, int T, int H, int N, bool varlen) {
     const bool split = splits_values(B, H, N, varlen);
     // stored segment states, then each workgroup's scratch, then (value columns split over two workgroups) the two
     // parts' sums of the five [token][key] gradients
-    return (rec_records(B, T, H, seg, varlen) + rec_areas(B, H, varlen) * (split ? 2 : 1) * seg) * state +
+    return (rec_records(B, T, H, seg, varlen) + rec_areas(B, H, varlen) * seg) * state +
            (split ? (size_t)2 * 5 * B * T * H * N * 4 : 0);
 }
 
-template <typename T, int N, int VS = 1>
-__global__ __launch_bounds__(256)
+template <typename T, int N, int VS = 1, int W = 4>
+__global__ __launch_bounds__(64 * W)
 void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, const T* __restrict__ k,
                           const T* __restrict__ v, const T* __restrict__ a, const T* __restrict__ b,
                           const T* __restrict__ d_o, const float* __restrict__ d_ht,
@@ -107,11 +116,12 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
     // ((first row >> cu_shift) + b + s (SEG >> cu_shift)) H + h): cu_shift 4 for the records of the chunked float32
     // backward, log2(SEG) for this backward's own forward pass.  The grid may be smaller than n_bh: a workgroup takes
     // every gridDim.x-th (sequence, head) and owns one scratch area.
-    constexpr int CPW = RecShape<N, VS>::CPW, SEG = RecShape<N, VS>::SEG;
+    typedef RecShape<N, VS, W> Shape;
+    constexpr int CPW = Shape::CPW, SEG = Shape::SEG, KEEP = Shape::KEEP, RB_TB = Shape::RB, NT = 64 * W;
+    static_assert(RB_TB % KEEP == 0 && SEG % RB_TB == 0, "kept states at multiples of KEEP in every block");
     constexpr int VQ = CPW / 4;                  // lanes across a wave's columns, four columns each
     constexpr int ROWS = N / (64 / VQ);          // state rows per lane
-    constexpr int PARTS = N / VS / CPW;          // waves
-    static_assert(PARTS == 4, "four waves per workgroup");
+    constexpr int PARTS = W;                     // waves
     // staged per-token vectors of one block, as float: a, d, b, k, v (both passes), r, do, dfac (reverse pass)
     enum { Q_A = 0, Q_D, Q_B, Q_K, Q_V, Q_R, Q_DO, Q_DF, Q_COUNT };
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -125,7 +135,7 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
     const int tid = threadIdx.x;
     if (run_if_any != nullptr) {
         int mine = 0;
-        for (int i = tid; i < n_flags; i += 256) mine |= run_if_any[i];
+        for (int i = tid; i < n_flags; i += NT) mine |= run_if_any[i];
         if (__syncthreads_or(mine) == 0) return;
     }
     const int lane = tid & 63;
@@ -133,7 +143,7 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
     const int ks = lane / VQ, vq = lane % VQ;
     const int row0 = ROWS * ks;                  // this lane's first state row
     const int64_t step = (int64_t)H * N;
-    float* my_scr = scratch + (int64_t)blockIdx.x * SEG * (N * N);
+    float* my_scr = scratch + (int64_t)(blockIdx.x / VS) * (SEG / KEEP) * (N * N);     // (the parts of a head share an area)
   for (int item = blockIdx.x; item < n_bh * VS; item += gridDim.x) {
     const int bh = item / VS, vs = item % VS;
     const int col0 = (N / VS) * vs + CPW * wave + 4 * vq;    // this lane's four value columns
@@ -153,40 +163,59 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
                                          : ckpt + (int64_t)bh * ckpt_per_head * (N * N);
     const int64_t ckpt_stride = cu != nullptr ? (int64_t)(SEG >> cu_shift) * H * (N * N) : (int64_t)ckpt_step * (N * N);
 
-    // one block of per-token vectors -> LDS as float (w as the decay d, and as dfac = dd/dw = -exp(w) d)
-    auto stage_block = [&](int t0, int nt, bool reverse_pass) {
-        for (int idx = tid; idx < RB_TB * (N / 4); idx += 256) {
-            const int tt = idx / (N / 4), e0 = (idx % (N / 4)) * 4;
-            if (tt >= nt) continue;
-            const int64_t off = base + (int64_t)(t0 + tt) * step + e0;
-            float x[4];
-            Io<T>::load4(a + off, x);
-            *reinterpret_cast<float4_t*>(&stage[Q_A][tt][e0]) = float4_t{x[0], x[1], x[2], x[3]};
-            Io<T>::load4(b + off, x);
-            *reinterpret_cast<float4_t*>(&stage[Q_B][tt][e0]) = float4_t{x[0], x[1], x[2], x[3]};
-            Io<T>::load4(k + off, x);
-            *reinterpret_cast<float4_t*>(&stage[Q_K][tt][e0]) = float4_t{x[0], x[1], x[2], x[3]};
-            Io<T>::load4(v + off, x);
-            *reinterpret_cast<float4_t*>(&stage[Q_V][tt][e0]) = float4_t{x[0], x[1], x[2], x[3]};
-            Io<T>::load4(w + off, x);
-            float dd[4], df[4];
+    // One block of per-token vectors -> LDS as float (w as the decay d, and as dfac = dd/dw = -exp(w) d), in two
+    // halves: request() asks for the block while the block before it is being computed, deposit() converts what
+    // has arrived.  reverse_pass adds r, do and dfac.
+    typedef T tvec4 __attribute__((ext_vector_type(4)));
+    constexpr int ITEMS = (RB_TB * (N / 4) + NT - 1) / NT;    // (token, four channels) items per thread
+    tvec4 raw[ITEMS][7];                                      // a, b, k, v, w, r, do
+    auto request = [&](int t0, int nt, bool reverse_pass) {
 #pragma unroll
-            for (int m = 0; m < 4; ++m) {
-                const float ew = __expf(x[m]);
-                dd[m] = __expf(-ew);
-                df[m] = -ew * dd[m];
-            }
-            *reinterpret_cast<float4_t*>(&stage[Q_D][tt][e0]) = float4_t{dd[0], dd[1], dd[2], dd[3]};
+        for (int it = 0; it < ITEMS; ++it) {
+            const int idx = it * NT + tid;
+            const int tt = idx / (N / 4), e0 = (idx % (N / 4)) * 4;
+            if (idx >= RB_TB * (N / 4) || tt >= nt) continue;
+            const int64_t off = base + (int64_t)(t0 + tt) * step + e0;
+            raw[it][0] = *reinterpret_cast<const tvec4*>(a + off);
+            raw[it][1] = *reinterpret_cast<const tvec4*>(b + off);
+            raw[it][2] = *reinterpret_cast<const tvec4*>(k + off);
+            raw[it][3] = *reinterpret_cast<const tvec4*>(v + off);
+            raw[it][4] = *reinterpret_cast<const tvec4*>(w + off);
             if (reverse_pass) {
-                *reinterpret_cast<float4_t*>(&stage[Q_DF][tt][e0]) = float4_t{df[0], df[1], df[2], df[3]};
-                Io<T>::load4(r + off, x);
-                *reinterpret_cast<float4_t*>(&stage[Q_R][tt][e0]) = float4_t{x[0], x[1], x[2], x[3]};
-                if (d_o != nullptr) Io<T>::load4(d_o + off, x);
-                else x[0] = x[1] = x[2] = x[3] = 0.f;
-                *reinterpret_cast<float4_t*>(&stage[Q_DO][tt][e0]) = float4_t{x[0], x[1], x[2], x[3]};
+                raw[it][5] = *reinterpret_cast<const tvec4*>(r + off);
+                if (d_o != nullptr) raw[it][6] = *reinterpret_cast<const tvec4*>(d_o + off);
             }
         }
     };
+    auto deposit = [&](int nt, bool reverse_pass) {
+        auto as_float = [](const tvec4& x) { return float4_t{(float)x[0], (float)x[1], (float)x[2], (float)x[3]}; };
+#pragma unroll
+        for (int it = 0; it < ITEMS; ++it) {
+            const int idx = it * NT + tid;
+            const int tt = idx / (N / 4), e0 = (idx % (N / 4)) * 4;
+            if (idx >= RB_TB * (N / 4) || tt >= nt) continue;
+            *reinterpret_cast<float4_t*>(&stage[Q_A][tt][e0]) = as_float(raw[it][0]);
+            *reinterpret_cast<float4_t*>(&stage[Q_B][tt][e0]) = as_float(raw[it][1]);
+            *reinterpret_cast<float4_t*>(&stage[Q_K][tt][e0]) = as_float(raw[it][2]);
+            *reinterpret_cast<float4_t*>(&stage[Q_V][tt][e0]) = as_float(raw[it][3]);
+            const float4_t w4 = as_float(raw[it][4]);
+            float4_t dd, df;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const float ew = __expf(w4[m]);
+                dd[m] = __expf(-ew);
+                df[m] = -ew * dd[m];
+            }
+            *reinterpret_cast<float4_t*>(&stage[Q_D][tt][e0]) = dd;
+            if (reverse_pass) {
+                *reinterpret_cast<float4_t*>(&stage[Q_DF][tt][e0]) = df;
+                *reinterpret_cast<float4_t*>(&stage[Q_R][tt][e0]) = as_float(raw[it][5]);
+                *reinterpret_cast<float4_t*>(&stage[Q_DO][tt][e0]) =
+                    d_o != nullptr ? as_float(raw[it][6]) : float4_t{0.f, 0.f, 0.f, 0.f};
+            }
+        }
+    };
+    auto block_len = [](int slen, int t0) { return slen - t0 < RB_TB ? slen - t0 : RB_TB; };
     auto rows_of = [&](int q, int tt, float (&x)[ROWS]) {
 #pragma unroll
         for (int i = 0; i < ROWS; i += 4) {
@@ -207,9 +236,11 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
         for (int i = 0; i < ROWS; ++i) Hd[i] = float4_t{0.f, 0.f, 0.f, 0.f};
     }
 
+    if (nseg > 0) request((nseg - 1) * SEG, block_len(T_len - (nseg - 1) * SEG, 0), false);
     for (int seg = nseg - 1; seg >= 0; --seg) {
         const int s0 = seg * SEG;
         const int slen = T_len - s0 < SEG ? T_len - s0 : SEG;
+        const int nblk = (slen + RB_TB - 1) / RB_TB;
         // ---- the segment forward once more: the state before each token -> scratch, sa -> LDS
         {
             float4_t s[ROWS];
@@ -219,19 +250,23 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
             for (int t0 = 0; t0 < slen; t0 += RB_TB) {
                 const int nt = slen - t0 < RB_TB ? slen - t0 : RB_TB;
                 __syncthreads();                 // the block before this one has been consumed
-                stage_block(s0 + t0, nt, false);
+                deposit(nt, false);
                 __syncthreads();
+                if (t0 + RB_TB < slen) request(s0 + t0 + RB_TB, block_len(slen, t0 + RB_TB), false);
+                else request(s0 + t0, nt, true);                       // the walk back starts with this block
+#pragma unroll 4
                 for (int tt = 0; tt < nt; ++tt) {
                     float av[ROWS], d[ROWS], bv[ROWS], kv[ROWS];
                     rows_of(Q_A, tt, av); rows_of(Q_D, tt, d); rows_of(Q_B, tt, bv); rows_of(Q_K, tt, kv);
                     const float4_t v4 = cols_of(Q_V, tt);
-                    float* dst = my_scr + (int64_t)(t0 + tt) * (N * N) + tile;
                     float4_t sa = {0.f, 0.f, 0.f, 0.f};
+                    if (KEEP == 1 || tt % KEEP == 0) {
+                        float* dst = my_scr + (int64_t)((t0 + tt) / KEEP) * (N * N) + tile;
 #pragma unroll
-                    for (int i = 0; i < ROWS; ++i) {
-                        *reinterpret_cast<float4_t*>(dst + i * N) = s[i];
-                        sa += av[i] * s[i];
+                        for (int i = 0; i < ROWS; ++i) *reinterpret_cast<float4_t*>(dst + i * N) = s[i];
                     }
+#pragma unroll
+                    for (int i = 0; i < ROWS; ++i) sa += av[i] * s[i];
                     sa.x = reduce_rows<VQ>(sa.x); sa.y = reduce_rows<VQ>(sa.y);
                     sa.z = reduce_rows<VQ>(sa.z); sa.w = reduce_rows<VQ>(sa.w);
                     if (ks == 0) *reinterpret_cast<float4_t*>(&sa_buf[t0 + tt][col0]) = sa;
@@ -240,20 +275,26 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
                 }
             }
         }
-        // ---- the segment backwards, block by block (the last, possibly short, block first)
-        const int nblk = (slen + RB_TB - 1) / RB_TB;
+        // ---- the segment backwards, block by block (the last, possibly short, block first).  A lane reads back
+        // the kept states that it wrote itself, each one group ahead of its use.
+        float4_t hk[ROWS];
+        auto fetch_kept = [&](int t) {
+            const float* src = my_scr + (int64_t)(t / KEEP) * (N * N) + tile;
+#pragma unroll
+            for (int i = 0; i < ROWS; ++i) hk[i] = *reinterpret_cast<const float4_t*>(src + i * N);
+        };
+        fetch_kept((slen - 1) / KEEP * KEEP);
         for (int blk = nblk - 1; blk >= 0; --blk) {
             const int t0 = blk * RB_TB;
             const int nt = slen - t0 < RB_TB ? slen - t0 : RB_TB;
             __syncthreads();                     // the block before: vectors consumed, partial sums written out;
                                                  // first block of the segment: the scratch stores above are done
-            stage_block(s0 + t0, nt, true);
+            deposit(nt, true);
             __syncthreads();
-            for (int tt = nt - 1; tt >= 0; --tt) {
-                float4_t hp[ROWS];               // the state before this token
-                const float* src = my_scr + (int64_t)(t0 + tt) * (N * N) + tile;
-#pragma unroll
-                for (int i = 0; i < ROWS; ++i) hp[i] = *reinterpret_cast<const float4_t*>(src + i * N);
+            if (blk > 0) request(s0 + t0 - RB_TB, RB_TB, true);
+            else if (seg > 0) request(s0 - SEG, RB_TB, false);          // the segment before this one: its first block
+            // one token backwards; hp: the state before it
+            auto reverse_step = [&](int tt, const float4_t (&hp)[ROWS]) {
                 float av[ROWS], d[ROWS], bv[ROWS], kv[ROWS], rv[ROWS];
                 rows_of(Q_A, tt, av); rows_of(Q_D, tt, d); rows_of(Q_B, tt, bv); rows_of(Q_K, tt, kv); rows_of(Q_R, tt, rv);
                 const float4_t v4 = cols_of(Q_V, tt), do4 = cols_of(Q_DO, tt);
@@ -293,26 +334,50 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
                     }
                     Hd[i] = d[i] * Hd[i] + av[i] * dsa4;
                 }
+            };
+            // a group of KEEP tokens (whole: without a branch between its steps), the last token first
+            auto walk_group = [&](int tg, int ng, auto whole) {
+                constexpr bool WHOLE = decltype(whole)::value;
+                float4_t hs[KEEP][ROWS];         // the states before the group's tokens: the first was kept
+#pragma unroll
+                for (int i = 0; i < ROWS; ++i) hs[0][i] = hk[i];
+                if (t0 + tg >= KEEP) fetch_kept(t0 + tg - KEEP);         // the group before, one group ahead
+#pragma unroll
+                for (int j = 1; j < KEEP; ++j) {
+                    if (!WHOLE && j >= ng) break;
+                    float d[ROWS], bv[ROWS], kv[ROWS];
+                    rows_of(Q_D, tg + j - 1, d); rows_of(Q_B, tg + j - 1, bv); rows_of(Q_K, tg + j - 1, kv);
+                    const float4_t v4 = cols_of(Q_V, tg + j - 1);
+                    const float4_t sa4 = *reinterpret_cast<const float4_t*>(&sa_buf[t0 + tg + j - 1][col0]);
+#pragma unroll
+                    for (int i = 0; i < ROWS; ++i) hs[j][i] = d[i] * hs[j - 1][i] + bv[i] * sa4 + kv[i] * v4;
+                }
+#pragma unroll
+                for (int j = KEEP - 1; j >= 0; --j)
+                    if (WHOLE || j < ng) reverse_step(tg + j, hs[j]);
+            };
+            for (int grp = (nt - 1) / KEEP; grp >= 0; --grp) {
+                const int tg = grp * KEEP;
+                if (nt - tg >= KEEP) walk_group(tg, KEEP, std::true_type{});
+                else walk_group(tg, nt - tg, std::false_type{});
             }
             __syncthreads();
-            // the five output rows of the block's tokens: sum over the four waves, four channels per thread
-            for (int idx = tid; idx < nt * (N / 4); idx += 256) {
-                const int tt = idx / (N / 4), e0 = (idx % (N / 4)) * 4;
+            // the five output rows of the block's tokens: sum over the waves, four channels of one output per thread
+            for (int idx = tid; idx < O_COUNT * nt * (N / 4); idx += NT) {
+                const int q = idx / (nt * (N / 4)), rem = idx % (nt * (N / 4));
+                const int tt = rem / (N / 4), e0 = (rem % (N / 4)) * 4;
                 const int64_t off = base + (int64_t)(s0 + t0 + tt) * step + e0;
-                T* const outs[O_COUNT] = {dr, dk, db, dw, da};
+                float4_t sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int q = 0; q < O_COUNT; ++q) {
-                    float4_t sum = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int p = 0; p < PARTS; ++p) sum += *reinterpret_cast<const float4_t*>(&part[q][tt][p][e0]);
-                    if (q == O_DD) sum = sum * *reinterpret_cast<const float4_t*>(&stage[Q_DF][tt][e0]);
-                    if constexpr (VS > 1) {
-                        const int64_t all = (int64_t)(n_bh / H) * T_rows * step;       // elements of one tensor
-                        *reinterpret_cast<float4_t*>(pbuf + ((int64_t)vs * O_COUNT + q) * all + off) = sum;
-                    } else {
-                        const float o4[4] = {sum.x, sum.y, sum.z, sum.w};
-                        Io<T>::store4(outs[q] + off, o4);
-                    }
+                for (int p = 0; p < PARTS; ++p) sum += *reinterpret_cast<const float4_t*>(&part[q][tt][p][e0]);
+                if (q == O_DD) sum = sum * *reinterpret_cast<const float4_t*>(&stage[Q_DF][tt][e0]);
+                if constexpr (VS > 1) {
+                    const int64_t all = (int64_t)(n_bh / H) * T_rows * step;           // elements of one tensor
+                    *reinterpret_cast<float4_t*>(pbuf + ((int64_t)vs * O_COUNT + q) * all + off) = sum;
+                } else {
+                    T* const out = q == O_DR ? dr : q == O_DK ? dk : q == O_DB ? db : q == O_DD ? dw : da;
+                    const float o4[4] = {sum.x, sum.y, sum.z, sum.w};
+                    Io<T>::store4(out + off, o4);
                 }
             }
         }
@@ -346,22 +411,23 @@ void bwd_recurrent_combine_kernel(const float* __restrict__ pbuf, T* __restrict_
 }
 
 namespace {
-template <int N> constexpr size_t rec_lds_bytes() {
-    return sizeof(float) * ((size_t)8 * RB_TB * N + (size_t)RecShape<N>::SEG * N + (size_t)5 * RB_TB * 4 * N);
+template <int N, int VS, int W> constexpr size_t rec_lds_bytes() {
+    typedef RecShape<N, VS, W> Shape;
+    return sizeof(float) * ((size_t)8 * Shape::RB * N + (size_t)Shape::SEG * N + (size_t)5 * Shape::RB * W * N);
 }
 
-template <typename T, int N, int VS = 1>
+template <typename T, int N, int VS = 1, int W = 4>
 hipError_t launch_bwd_rec_t(const BwdArgs& p, const float* ckpt, float* scratch, hipStream_t stream,
                             int ckpt_per_head = 0, int ckpt_step = 1, const int* run_if_any = nullptr, int n_flags = 0,
                             int max_grid = 0, int cu_shift = 4, float* pbuf = nullptr) {
     if (ckpt_per_head == 0) ckpt_per_head = (p.T + RecShape<N>::SEG - 1) / RecShape<N>::SEG;
     const int n_bh = p.B * p.H;
     const int grid = max_grid > 0 && n_bh > max_grid ? max_grid : n_bh * VS;
-    constexpr size_t lds = rec_lds_bytes<N>();
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_recurrent_kernel<T, N, VS>),
+    constexpr size_t lds = rec_lds_bytes<N, VS, W>();
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(bwd_recurrent_kernel<T, N, VS, W>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
-    bwd_recurrent_kernel<T, N, VS><<<dim3((unsigned)grid), dim3(256), lds, stream>>>(
+    bwd_recurrent_kernel<T, N, VS, W><<<dim3((unsigned)grid), dim3(64 * W), lds, stream>>>(
         (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, (const T*)p.a, (const T*)p.b,
         (const T*)p.dO, p.dht, ckpt, scratch, (T*)p.dr, (T*)p.dw, (T*)p.dk, (T*)p.dv, (T*)p.da, (T*)p.db,
         p.dh0, p.T, p.H, ckpt_per_head, ckpt_step, run_if_any, n_flags, p.cu, n_bh, cu_shift, pbuf);
@@ -408,18 +474,18 @@ hipError_t launch_bwd_recurrent(const BwdArgs& p, int N, void* ws, hipStream_t s
     // packed: the records lie by slots of one per segment, and at most WALK_MAX_GRID workgroups walk
     const int grid = varlen ? WALK_MAX_GRID : 0, shift = seg == 64 ? 6 : 5;
     if (splits_values(p.B, p.H, N, varlen)) {
-        float* pbuf = scratch + (size_t)p.B * p.H * 2 * seg * N * N;
-        return p.dtype == RWKV7_DTYPE_BF16  ? launch_bwd_rec_t<bf16_t, 128, 2>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, 0, shift, pbuf)
-               : p.dtype == RWKV7_DTYPE_F16 ? launch_bwd_rec_t<f16_t, 128, 2>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, 0, shift, pbuf)
-                                            : launch_bwd_rec_t<float, 128, 2>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, 0, shift, pbuf);
+        float* pbuf = scratch + (size_t)p.B * p.H * seg * N * N;
+        return p.dtype == RWKV7_DTYPE_BF16  ? launch_bwd_rec_t<bf16_t, 128, 2, W_SPLIT>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, 0, shift, pbuf)
+               : p.dtype == RWKV7_DTYPE_F16 ? launch_bwd_rec_t<f16_t, 128, 2, W_SPLIT>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, 0, shift, pbuf)
+                                            : launch_bwd_rec_t<float, 128, 2, W_SPLIT>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, 0, shift, pbuf);
     }
     if (N == 128)
-        return p.dtype == RWKV7_DTYPE_BF16  ? launch_bwd_rec_t<bf16_t, 128>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)
-               : p.dtype == RWKV7_DTYPE_F16 ? launch_bwd_rec_t<f16_t, 128>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)
-                                            : launch_bwd_rec_t<float, 128>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift);
-    return p.dtype == RWKV7_DTYPE_BF16  ? launch_bwd_rec_t<bf16_t, 64>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)
-           : p.dtype == RWKV7_DTYPE_F16 ? launch_bwd_rec_t<f16_t, 64>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)
-                                        : launch_bwd_rec_t<float, 64>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift);
+        return p.dtype == RWKV7_DTYPE_BF16  ? launch_bwd_rec_t<bf16_t, 128, 1, W_128>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)
+               : p.dtype == RWKV7_DTYPE_F16 ? launch_bwd_rec_t<f16_t, 128, 1, W_128>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)
+                                            : launch_bwd_rec_t<float, 128, 1, W_128>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift);
+    return p.dtype == RWKV7_DTYPE_BF16  ? launch_bwd_rec_t<bf16_t, 64, 1, W_64>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)
+           : p.dtype == RWKV7_DTYPE_F16 ? launch_bwd_rec_t<f16_t, 64, 1, W_64>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift)
+                                        : launch_bwd_rec_t<float, 64, 1, W_64>(p, ckpt, scratch, stream, 0, 1, nullptr, 0, grid, shift);
 }
 
 }  // namespace rwkv7

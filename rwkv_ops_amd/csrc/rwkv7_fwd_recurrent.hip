@@ -33,8 +33,10 @@ constexpr int REC_TB = 16;                       // tokens per staged block
 
 // V6 = true is the RWKV6 operator (/root/reference/rwkv_ops/rwkv6_kernel/ops_rwkv_kernel.py:65-73):
 // o = r^T (diag(u) k v^T + h),  h <- k v^T + diag(d) h, with u [H][N] passed in b's place and a unused.
-template <typename T, int N, bool V6 = false, int CPW = (N == 64 ? 16 : 32)>
-__global__ __launch_bounds__(64 * (N / CPW))
+// VS = 2: the value columns of a head over two workgroups (blockIdx.x = (batch, head) * 2 + half), for calls with
+// fewer heads than CUs; the columns being independent, the halves share nothing.
+template <typename T, int N, bool V6 = false, int VS = 1, int CPW = (N == 64 ? 16 : 32) / VS>
+__global__ __launch_bounds__(64 * (N / VS / CPW))
 void fwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, const T* __restrict__ k,
                           const T* __restrict__ v, const T* __restrict__ a, const T* __restrict__ b,
                           const float* __restrict__ h0, int64_t h0_batch_stride,
@@ -48,19 +50,20 @@ void fwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
     // the next sequence's), record (slot + t / seg) H + h; (T_total / seg + n_seq) H records in all.
     constexpr int VQ = CPW / 4;                  // lanes across a wave's columns, four columns each
     constexpr int ROWS = N / (64 / VQ);          // state rows per lane
-    constexpr int NT = 64 * (N / CPW);           // threads
+    constexpr int NT = 64 * (N / VS / CPW);      // threads
     constexpr int PER16 = 16 / (int)sizeof(T);   // elements per 16-byte load
     constexpr int PIECES = 6 * REC_TB * N / PER16 / NT;    // 16-byte loads per thread and block
     __shared__ __attribute__((aligned(16))) float stage[6][REC_TB][N];   // a, d, b, k, r, v
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int part = tid >> 6;                   // which CPW value columns
+    const int bh = blockIdx.x / VS;
+    const int col0 = (N / VS) * (blockIdx.x % VS) + CPW * (tid >> 6);    // the wave's first value column
     const int H = L.H;
-    const int bi = blockIdx.x / H, hi = blockIdx.x % H;
+    const int bi = bh / H, hi = bh % H;
     const SeqSpan sp = seq_span(L, bi);
     const int T_len = sp.len;
     const int ks = lane / VQ, vq = lane % VQ;
-    const int tile = (ROWS * ks) * N + CPW * part + 4 * vq;
+    const int tile = (ROWS * ks) * N + col0 + 4 * vq;
 
     float4_t s[ROWS];
     if (h0 != nullptr) {
@@ -135,7 +138,7 @@ void fwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
         if (seg_states != nullptr && t0 % seg == 0) {
             const int nseg = (T_len + seg - 1) / seg;
             const int64_t rec = L.cu != nullptr ? (sp.tok0 / seg + bi + t0 / seg) * H + hi
-                                                : (int64_t)blockIdx.x * nseg + t0 / seg;
+                                                : (int64_t)bh * nseg + t0 / seg;
             float* dst = seg_states + rec * (N * N) + tile;
 #pragma unroll
             for (int i = 0; i < ROWS; ++i) *reinterpret_cast<float4_t*>(dst + i * N) = s[i];
@@ -154,13 +157,18 @@ void fwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
 #pragma unroll
                 for (int m = 0; m < 4; ++m) { av[i + m] = a4[m]; d[i + m] = d4[m]; bv[i + m] = b4[m]; kv[i + m] = k4[m]; rv[i + m] = r4[m]; }
             }
-            const float4_t v4 = *reinterpret_cast<const float4_t*>(&stage[5][tt][CPW * part + 4 * vq]);
+            const float4_t v4 = *reinterpret_cast<const float4_t*>(&stage[5][tt][col0 + 4 * vq]);
             float4_t sa = {0.f, 0.f, 0.f, 0.f};
             if constexpr (!V6) {
 #pragma unroll
                 for (int i = 0; i < ROWS; ++i) sa += av[i] * s[i];
                 sa.x = reduce_row_groups<VQ>(sa.x); sa.y = reduce_row_groups<VQ>(sa.y);
                 sa.z = reduce_row_groups<VQ>(sa.z); sa.w = reduce_row_groups<VQ>(sa.w);
+            }
+            if (!V6 && o == nullptr) {                  // the states only
+#pragma unroll
+                for (int i = 0; i < ROWS; ++i) s[i] = d[i] * s[i] + bv[i] * sa + kv[i] * v4;
+                continue;
             }
             float4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -178,31 +186,40 @@ void fwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
             acc.z = reduce_row_groups<VQ>(acc.z); acc.w = reduce_row_groups<VQ>(acc.w);
             if (ks == 0 && o != nullptr) {
                 const float ov[4] = {acc.x, acc.y, acc.z, acc.w};
-                Io<T>::store4(o + base + (t0 + tt) * step + CPW * part + 4 * vq, ov);
+                Io<T>::store4(o + base + (t0 + tt) * step + col0 + 4 * vq, ov);
             }
         }
     }
     if (ht != nullptr) {
-        float* dst = ht + (int64_t)blockIdx.x * (N * N) + tile;
+        float* dst = ht + (int64_t)bh * (N * N) + tile;
 #pragma unroll
         for (int i = 0; i < ROWS; ++i) *reinterpret_cast<float4_t*>(dst + i * N) = s[i];
     }
 }
 
+// head size 128 and fewer (batch, head) pairs than CUs: two workgroups per pair
+constexpr int VSPLIT_MAX_BH = 192;
+
 template <typename T, int N>
-static hipError_t launch_t(const SeqArgs& p, hipStream_t stream) {
-    fwd_recurrent_kernel<T, N><<<dim3((unsigned)(p.B * p.H)), dim3(256), 0, stream>>>(
-        (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, (const T*)p.a, (const T*)p.b,
-        p.h0, p.h0_batch_stride, p.h0_map, p.n_state, (T*)p.o, p.ht, seq_layout(p, nullptr));
+static hipError_t launch_t(const SeqArgs& p, hipStream_t stream, float* states = nullptr, int seg = 0) {
+    const int n_bh = p.B * p.H;
+    T* o = states != nullptr ? nullptr : (T*)p.o;
+    float* ht = states != nullptr ? nullptr : p.ht;
+    const int* map = states != nullptr ? nullptr : p.h0_map;
+    if (N == 128 && n_bh <= VSPLIT_MAX_BH)
+        fwd_recurrent_kernel<T, N, false, N == 128 ? 2 : 1><<<dim3((unsigned)(2 * n_bh)), dim3(256), 0, stream>>>(
+            (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, (const T*)p.a, (const T*)p.b,
+            p.h0, p.h0_batch_stride, map, p.n_state, o, ht, seq_layout(p, nullptr), states, seg);
+    else
+        fwd_recurrent_kernel<T, N><<<dim3((unsigned)n_bh), dim3(256), 0, stream>>>(
+            (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, (const T*)p.a, (const T*)p.b,
+            p.h0, p.h0_batch_stride, map, p.n_state, o, ht, seq_layout(p, nullptr), states, seg);
     return hipGetLastError();
 }
 
 template <typename T, int N>
 static hipError_t launch_states_t(const SeqArgs& p, float* states, int seg, hipStream_t stream) {
-    fwd_recurrent_kernel<T, N><<<dim3((unsigned)(p.B * p.H)), dim3(256), 0, stream>>>(
-        (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, (const T*)p.a, (const T*)p.b,
-        p.h0, p.h0_batch_stride, nullptr, 0, nullptr, nullptr, seq_layout(p, nullptr), states, seg);
-    return hipGetLastError();
+    return launch_t<T, N>(p, stream, states, seg);
 }
 
 // the forward without outputs, storing the state at the start of every segment of `seg` tokens (dense batches, or
