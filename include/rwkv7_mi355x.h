@@ -90,7 +90,7 @@ const char* rwkv7_status_string(int status);
  * rwkv7_fwd, rwkv7_fwd_gather, rwkv7_fwd_varlen, rwkv7_fwd_noalloc, rwkv7_fwd_recurrent, the two decode-step
  * calls and rwkv7_bwd_recurrent.  bf16 with T > 12 runs a chunked MFMA kernel of its own (one workgroup per
  * (batch, head) walking the chunks with the state in registers; no workspace, ws may be NULL); float32, float16
- * and T <= 12 run the float32 recurrent kernel at this head size (about 1 us per token).  rwkv7_bwd answers
+ * and T <= 12 run the float32 recurrent kernel at this head size (0.5 to 1 us per token).  rwkv7_bwd answers
  * RWKV7_ERR_BAD_HEAD_SIZE for it: its gradients come from rwkv7_bwd_recurrent. */
 size_t rwkv7_fwd_workspace_bytes(int B, int T, int H, int dtype);
 int rwkv7_fwd(const void* r, const void* w, const void* k, const void* v,
@@ -224,10 +224,11 @@ int rwkv7_bwd(const void* r, const void* w, const void* k, const void* v,
  * framework's autograd) one token at a time in float32 arithmetic, for either dtype of the tensors
  * (bf16, f32, f16: values are widened on load, gradients rounded on store) and K = V = 64 or 128: the
  * token-by-token path -- head size 128, float16, float32 calls of a dozen tokens or with very strong decays --
- * several microseconds per token, not the throughput path.  Same arguments and meaning as rwkv7_bwd; dense batches only.  The workspace
- * (rwkv7_bwd_recurrent_workspace_bytes: the state of every (batch, head) at the start of each 64-token
- * segment (32 tokens for K = 128), plus one segment's worth of per-token states per (batch, head)) grows
- * with B*H*T*K*V / 16. */
+ * two to three microseconds per token, not the throughput path.  Same arguments and meaning as rwkv7_bwd; dense
+ * batches only.  The workspace (rwkv7_bwd_recurrent_workspace_bytes: the state of every (batch, head) at the start
+ * of each 64-token segment (32 tokens for K = 128), plus one segment's worth of per-token states per (batch, head))
+ * grows with B*H*T*K*V / 16.  K = 128 with at most 192 (batch, head) pairs splits the value columns of a head
+ * over two workgroups and adds 40 bytes per element of a [B,T,H,K] tensor for their partial sums. */
 size_t rwkv7_bwd_recurrent_workspace_bytes(int B, int T, int H, int K);
 int rwkv7_bwd_recurrent(const void* r, const void* w, const void* k, const void* v,
                         const void* a, const void* b,
