@@ -43,7 +43,10 @@ def run(lib, device, xs, dO, dS, N, dtype, entry="rwkv7_bwd_recurrent"):
     (64, torch.float32, 2, 1, 2), (64, torch.float32, 1, 7, 1), (64, torch.float32, 2, 63, 2), (64, torch.float32, 1, 64, 3),
     (64, torch.float32, 2, 65, 1), (64, torch.float32, 1, 200, 2), (64, torch.bfloat16, 2, 130, 2), (64, torch.float16, 1, 77, 2),
     (128, torch.float32, 1, 1, 1), (128, torch.float32, 2, 33, 2), (128, torch.float32, 1, 100, 1), (128, torch.bfloat16, 1, 64, 2),
-    (128, torch.float16, 2, 40, 1)])
+    (128, torch.float16, 2, 40, 1),
+    # (every fourth state is kept and a block holds 4 or 8 tokens: lengths around those multiples)
+    (128, torch.float32, 1, 2, 1), (128, torch.float32, 1, 3, 2), (128, torch.float32, 2, 35, 1), (128, torch.bfloat16, 1, 6, 1),
+    (64, torch.float32, 1, 2, 1), (64, torch.float32, 2, 3, 1), (64, torch.float32, 1, 9, 2), (64, torch.float32, 1, 70, 1)])
 def test_recurrent_backward_matches_oracle_autograd(device, N, dtype, B, T, H):
     lib = _lib.load()
     xs = make_inputs(B, T, H, N, seed=3000 + T + N, dtype=dtype)
