@@ -90,8 +90,10 @@ const char* rwkv7_status_string(int status);
  * rwkv7_fwd, rwkv7_fwd_gather, rwkv7_fwd_varlen, rwkv7_fwd_noalloc, rwkv7_fwd_recurrent, the two decode-step
  * calls and rwkv7_bwd_recurrent.  bf16 with T > 12 runs a chunked MFMA kernel of its own (one workgroup per
  * (batch, head) walking the chunks with the state in registers; no workspace, ws may be NULL); float32, float16
- * and T <= 12 run the float32 recurrent kernel at this head size (0.5 to 1 us per token).  rwkv7_bwd answers
- * RWKV7_ERR_BAD_HEAD_SIZE for it: its gradients come from rwkv7_bwd_recurrent. */
+ * and T <= 12 run the float32 recurrent kernel at this head size (0.5 to 1 us per token).  rwkv7_bwd and
+ * rwkv7_bwd_varlen hand a call at this head size to rwkv7_bwd_recurrent / rwkv7_bwd_recurrent_varlen (any of the
+ * three dtypes), whose workspace sizes apply: rwkv7_bwd_recurrent_workspace_bytes(B, T, H, 128) and
+ * rwkv7_bwd_recurrent_varlen_workspace_bytes(n_seq, T_total, H, 128). */
 size_t rwkv7_fwd_workspace_bytes(int B, int T, int H, int dtype);
 int rwkv7_fwd(const void* r, const void* w, const void* k, const void* v,
               const void* a, const void* b,
@@ -275,8 +277,8 @@ int rwkv7_bwd_varlen(const void* r, const void* w, const void* k, const void* v,
                      int T_total, int H, int K, int V, int dtype,
                      void* ws, size_t ws_bytes, void* stream);
 /* rwkv7_bwd_recurrent over packed sequences: the token-by-token float32 backward (bf16, f32 or f16 tensors,
- * K = V = 64 or 128) with the arguments of rwkv7_bwd_varlen -- the gradients of packed rows at head size 128, which
- * rwkv7_bwd_varlen does not take.  No counterpart in the reference, like the packed calls above.  Workspace: one
+ * K = V = 64 or 128) with the arguments of rwkv7_bwd_varlen -- what rwkv7_bwd_varlen runs for packed rows at head
+ * size 128.  No counterpart in the reference, like the packed calls above.  Workspace: one
  * state per segment of 64 tokens (32 at K = 128) for T_total / segment + n_seq segments per head, plus a segment's
  * worth of states for each of at most 1024 (sequence, head) pairs walked at a time. */
 size_t rwkv7_bwd_recurrent_varlen_workspace_bytes(int n_seq, int T_total, int H, int K);

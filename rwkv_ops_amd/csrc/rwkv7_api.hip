@@ -59,7 +59,7 @@ const char* rwkv7_status_string(int status) {
         case RWKV7_OK: return "ok";
         case RWKV7_ERR_NULL_POINTER: return "a required pointer is NULL";
         case RWKV7_ERR_BAD_DTYPE: return "dtype must be RWKV7_DTYPE_BF16 (0), RWKV7_DTYPE_F32 (1) or RWKV7_DTYPE_F16 (2)";
-        case RWKV7_ERR_BAD_HEAD_SIZE: return "K = V = 64 (every entry point) or 128 (forward, decode step and rwkv7_bwd_recurrent) only";
+        case RWKV7_ERR_BAD_HEAD_SIZE: return "K = V = 64 (every entry point) or 128 (every entry point but the two-kernel ones and the RWKV6 operator) only";
         case RWKV7_ERR_BAD_SHAPE: return "B, T and H must be >= 1 and B*H*ceil(T/64) <= 2^30";
         case RWKV7_ERR_BAD_STRIDE: return "h0_batch_stride must be 0 (broadcast) or H*K*V";
         case RWKV7_ERR_WORKSPACE: return "workspace is NULL, not 256-byte aligned or too small";
@@ -313,8 +313,12 @@ int rwkv7_bwd(const void* r, const void* w, const void* k, const void* v, const 
               void* dr, void* dw, void* dk, void* dv, void* da, void* db, float* dh0,
               int B, int T, int H, int K, int V, int dtype, void* ws, size_t ws_bytes, void* stream)
 {
-    // float32 gradients (K = V = 64 here; rwkv7_bwd_recurrent takes 128 too): beyond a dozen tokens the chunked
-    // float32 backward, otherwise the token-by-token one
+    // head size 128 has the token-by-token backward only (every dtype; its own workspace size)
+    if (K == 128 && V == 128)
+        return rwkv7_bwd_recurrent(r, w, k, v, a, b, h0, h0_batch_stride, d_o, d_ht, dr, dw, dk, dv, da, db, dh0,
+                                   B, T, H, K, V, dtype, ws, ws_bytes, stream);
+    // float32 gradients at K = V = 64: beyond a dozen tokens the chunked float32 backward, otherwise the
+    // token-by-token one
     if (dtype == RWKV7_DTYPE_F32 && K == 64 && V == 64) {
         if (T <= RECURRENT_MAX_T)
             return rwkv7_bwd_recurrent(r, w, k, v, a, b, h0, h0_batch_stride, d_o, d_ht, dr, dw, dk, dv, da, db, dh0,
@@ -409,6 +413,9 @@ int rwkv7_bwd_varlen(const void* r, const void* w, const void* k, const void* v,
                      void* dr, void* dw, void* dk, void* dv, void* da, void* db, float* dh0,
                      int T_total, int H, int K, int V, int dtype, void* ws, size_t ws_bytes, void* stream)
 {
+    if (K == 128 && V == 128)           // head size 128: the token-by-token backward (its own workspace size)
+        return rwkv7_bwd_recurrent_varlen(r, w, k, v, a, b, cu_seqlens, n_seq, h0, h0_batch_stride, d_o, d_ht,
+                                          dr, dw, dk, dv, da, db, dh0, T_total, H, K, V, dtype, ws, ws_bytes, stream);
     // float32 tensors (K = V = 64): the chunked float32 backward over the packed sequences
     const bool f32 = dtype == RWKV7_DTYPE_F32 && K == 64 && V == 64;
     int rc = check_seq(r, w, k, v, a, b, h0, h0_batch_stride, dr, nullptr, 1, T_total, H, K, V, dtype);

@@ -60,10 +60,11 @@ def test_argument_errors_do_not_launch():
     assert _call_fwd(lib, ptrs=[0x1004] + [0x1000] * 5) == -7
     rc = lib.rwkv7_decode_step(*[0x1000] * 6, None, 0, 0x1000, None, 1, 1, 64, 32, 0, None)
     assert rc == -3
-    # K = V = 128 exists for the forward and the decode step only: the backward and the two-kernel entry
-    # points refuse it
+    # K = V = 128: the backward hands it to the token-by-token kernel (which asks for its workspace); the
+    # two-kernel entry points refuse it
     rc = lib.rwkv7_bwd(*[0x1000] * 6, None, 0, None, None, *[0x1000] * 6, None, 1, 4, 2, 128, 128, 0, None, 0, None)
-    assert rc == -3
+    assert rc == -6
+    assert lib.rwkv7_bwd_recurrent_workspace_bytes(1, 4, 2, 128) > 0
     rc = lib.rwkv7_fwd_chunk_summary(*[0x1000] * 6, 1, 4, 2, 128, 128, 0, None, 0, None)
     assert rc == -3
     assert _call_fwd(lib, K=256, V=256) == -3
@@ -108,7 +109,7 @@ def test_varlen_argument_errors_do_not_launch():
     assert lib.rwkv7_bwd_varlen_workspace_bytes(2000, 20000, 4, 1) < (20000 // 16 + 2000) * 4 * 40960 + 1025 * (1 << 20)
     rc = lib.rwkv7_bwd_varlen(*[0x1000] * 6, 0x3000, 2, None, 0, None, None, *[0x1000] * 6, None,
                               100, 2, 128, 128, 1, None, 0, None)
-    assert rc == -3                                      # ... at head size 64 only
+    assert rc == -6                                      # head size 128: the token-by-token backward's workspace
     rc = lib.rwkv7_bwd_varlen(*[0x1000] * 6, None, 2, None, 0, None, None, *[0x1000] * 6, None,
                               100, 2, 64, 64, 0, None, 0, None)
     assert rc == -1

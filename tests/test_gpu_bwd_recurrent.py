@@ -157,3 +157,44 @@ def test_recurrent_and_chunked_backward_agree(device):
     chk = run(lib, device, xs, dO, dS, N, torch.bfloat16, entry="rwkv7_bwd")
     for n, x, y in zip(GRAD_NAMES, chk, rec):
         assert rel_l2(x, y) < GRAD_TOL[n], n
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_rwkv7_bwd_takes_head_size_128(device, dtype):
+    """rwkv7_bwd and rwkv7_bwd_varlen at K = V = 128 are the token-by-token backward under their own names (with
+    its workspace size): the same bits as rwkv7_bwd_recurrent / rwkv7_bwd_recurrent_varlen."""
+    lib = _lib.load()
+    B, T, H, N = 2, 45, 2, 128
+    xs = make_inputs(B, T, H, N, seed=3600, dtype=dtype)
+    g = torch.Generator().manual_seed(7)
+    dO = torch.randn(B, T, H, N, generator=g).to(dtype)
+    dS = 0.1 * torch.randn(B, H, N, N, generator=g)
+    ref = run(lib, device, xs, dO, dS, N, dtype)
+    dev = [x.to(device) for x in xs[:6]]
+    h0, dO_d, dS_d = xs[6].to(device), dO.to(device), dS.to(device)
+    p = lambda t: None if t is None else t.data_ptr()
+    stream = torch.cuda.current_stream().cuda_stream
+    grads = [torch.full_like(dev[0], float("nan")) for _ in range(6)]
+    dh0 = torch.full((B, H, N, N), float("nan"), device=device)
+    size = lib.rwkv7_bwd_recurrent_workspace_bytes(B, T, H, N)
+    ws = torch.empty(size, dtype=torch.uint8, device=device)
+    args = (*[p(x) for x in dev], p(h0), H * N * N, p(dO_d), p(dS_d), *[p(x) for x in grads], p(dh0), B, T, H, N, N, CODE[dtype])
+    assert lib.rwkv7_bwd(*args, p(ws), size - 256, stream) == -6         # RWKV7_ERR_WORKSPACE
+    assert lib.rwkv7_bwd(*args, p(ws), size, stream) == 0
+    torch.cuda.synchronize()
+    for n, a_, b_ in zip(GRAD_NAMES, grads + [dh0], ref):
+        assert torch.equal(a_, b_), n
+    # the same rows as one packed row of B sequences
+    packed = [x.reshape(1, B * T, H, N) for x in dev]
+    cu = torch.tensor([0, T, 2 * T], dtype=torch.int32, device=device)
+    want = torch.ops.rwkv_ops_amd.rwkv7_bwd_recurrent_varlen(*packed, h0, dO_d.reshape(1, B * T, H, N), dS_d, cu)
+    grads = [torch.full_like(packed[0], float("nan")) for _ in range(6)]
+    dh0 = torch.full((B, H, N, N), float("nan"), device=device)
+    size = lib.rwkv7_bwd_recurrent_varlen_workspace_bytes(B, B * T, H, N)
+    ws = torch.empty(size, dtype=torch.uint8, device=device)
+    rc = lib.rwkv7_bwd_varlen(*[p(x) for x in packed], p(cu), B, p(h0), H * N * N, p(dO_d), p(dS_d), *[p(x) for x in grads],
+                              p(dh0), B * T, H, N, N, CODE[dtype], p(ws), size, stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    for n, a_, b_ in zip(GRAD_NAMES, grads + [dh0], want):
+        assert torch.equal(a_, b_), n
