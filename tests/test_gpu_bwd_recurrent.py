@@ -61,9 +61,10 @@ def test_recurrent_backward_matches_oracle_autograd(device, N, dtype, B, T, H):
         assert errs[n] < (1e-4 if n == "dh0" else TOL[dtype]), (n, errs)
 
 
-def test_recurrent_backward_variants(device):
+@pytest.mark.parametrize("N", [64, 128])
+def test_recurrent_backward_variants(device, N):
     lib = _lib.load()
-    B, T, H, N = 2, 90, 2, 64
+    B, T, H = 2, 90, 2
     xs = list(make_inputs(B, T, H, N, seed=3100, dtype=torch.float32))
     g = torch.Generator().manual_seed(3)
     dO = torch.randn(B, T, H, N, generator=g)
