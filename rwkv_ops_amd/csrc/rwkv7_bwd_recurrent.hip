@@ -12,17 +12,21 @@
 //     dk  = H v,   dv = H^T k,   db = H sa,   dd = rowsum(H * h),   dsa = H^T b
 //     da  = h dsa,   dw = dd * d * (-exp(w))
 //     H  <- diag(d) H + a dsa^T                    (adjoint of h)
-// The reverse walk needs h before every step.  Two launches:
+// The reverse walk needs h before every step.  Launches:
 //   1. the recurrent forward kernel (rwkv7_fwd_recurrent.hip) run once more, storing the state at the start of
 //      every segment of SEG tokens;
-//   2. bwd_recurrent_kernel, one workgroup per (batch, head), segments last to first: it re-runs the segment
-//      forward from its stored state, writing the state before each token to a per-workgroup scratch area (and
-//      sa to LDS), then walks the segment backwards.
+//   2. bwd_recurrent_kernel, one workgroup per (batch, head) (two at head size 128 when heads are few: VS below),
+//      segments last to first: it re-runs the segment forward from its stored state, writing the state before
+//      every KEEP-th token to a per-head scratch area (and sa of every token to LDS), then walks the segment
+//      backwards in groups of KEEP tokens -- the kept state, requested a group ahead, and KEEP - 1 steps forward
+//      from it;
+//   3. with VS = 2, bwd_recurrent_combine_kernel adds the two halves' sums of dr, dk, db, dw, da.
 // Layout: that of the forward kernel -- a wave owns CPW value columns, lane (ks, vq) holds ROWS rows of four of
-// them, for h and H alike.  Sums over K (sa, dv, dsa: the ones on the chain) are in-register plus the forward
-// kernel's cross-lane reduction inside the wave; sums over V (dr, dk, db, dd, da) cross the waves, but nothing
-// later depends on them, so each wave leaves its partial sums in LDS and the workgroup adds them up and writes
-// the five output rows once per block of RB_TB tokens.
+// them, for h and H alike; W = 4 waves, or 8 at head size 128 (two waves per SIMD: one wave alone issues a vector
+// instruction every 4 cycles, the SIMD takes one every 2).  Sums over K (sa, dv, dsa: the ones on the chain) are
+// in-register plus the forward kernel's cross-lane reduction inside the wave; sums over V (dr, dk, db, dd, da)
+// cross the waves, but nothing later depends on them, so each wave leaves its partial sums in LDS and the
+// workgroup adds them up and writes the five output rows once per block of RB tokens.
 #include <type_traits>
 #include "rwkv7_common.h"
 #include "rwkv7_kernels.h"
@@ -31,7 +35,6 @@
 namespace rwkv7 {
 
 namespace {
-
 
 template <int VQ>
 __device__ __forceinline__ float reduce_rows(float x) {      // sum over the lanes that share lane % VQ

@@ -4,11 +4,12 @@
 // one token at a time, all arithmetic in float32 whatever the input type.  The state stays in
 // registers for the whole sequence, laid out like the decode kernel's: the value columns are independent,
 // so one wave64 owns CPW of them (N / CPW waves per (batch, head), one workgroup); with VQ = CPW / 4, lane =
-// (ks = lane / VQ, vq = lane % VQ) holds N / (64 / VQ) rows of columns CPW*part + 4*vq .. +3; the two
+// (ks = lane / VQ, vq = lane % VQ) holds N / (64 / VQ) rows of columns CPW*wave + 4*vq .. +3; the two
 // contractions over K are in-register FMAs plus a cross-lane reduction over the 64 / VQ row groups (DPP
 // rotations and lane swaps, no LDS).  K = 64 runs with CPW = 16 (four waves per head, about 130 instructions
 // per wave and token: 0.46 us per token against 0.59 with CPW = 32), K = 128 with CPW = 32 (eight waves per
-// head were no faster for one sequence and slower for many).  The per-token vectors
+// head were no faster for one sequence and slower for many), or, when there are fewer (batch, head) pairs than
+// CUs, as two workgroups per pair with CPW = 16 and half of the value columns each.  The per-token vectors
 // come in blocks of 16 tokens: the workgroup requests a block with 16-byte loads while it computes the
 // block before it, then converts it to float32 into LDS (w already as the decay exp(-exp(w))), from
 // where every lane reads the entries of its rows.  What is left per token is the chain state -> a^T h ->
