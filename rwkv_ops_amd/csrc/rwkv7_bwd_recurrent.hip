@@ -36,13 +36,29 @@ namespace rwkv7 {
 
 namespace {
 
+// Sums over the lanes that share lane % VQ (the rows of the state that a wave holds): first inside a 16-lane row
 template <int VQ>
-__device__ __forceinline__ float reduce_rows(float x) {      // sum over the lanes that share lane % VQ
+__device__ __forceinline__ float reduce_rows_in_row(float x) {
     if constexpr (VQ == 2)
         x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x122, 0xf, 0xf, true));   // row_ror:2
     if constexpr (VQ <= 4)
         x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x124, 0xf, 0xf, true));   // row_ror:4
-    return sum_lane_groups_of_8(x);
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x128, 0xf, 0xf, true));       // row_ror:8
+    return x;
+}
+// then over the four rows, the four components of v at once (rwkv7_common.h), delivered to all lanes
+template <int VQ>
+__device__ __forceinline__ void reduce_rows4(float4_t& v) {
+    float a = reduce_rows_in_row<VQ>(v.x), b = reduce_rows_in_row<VQ>(v.y);
+    float c = reduce_rows_in_row<VQ>(v.z), d = reduce_rows_in_row<VQ>(v.w);
+    sum4_over_rows(a, b, c, d);
+    v = float4_t{a, b, c, d};
+}
+// ... delivered one component per 16-lane row: row r of the wave gets component r
+template <int VQ>
+__device__ __forceinline__ float reduce_rows4_scattered(const float4_t& v) {
+    return sum4_over_rows_scattered(reduce_rows_in_row<VQ>(v.x), reduce_rows_in_row<VQ>(v.y),
+                                    reduce_rows_in_row<VQ>(v.z), reduce_rows_in_row<VQ>(v.w));
 }
 
 // sum over the VQ adjacent lanes that share lane / VQ (the columns of one row group), delivered to lane % VQ == 0
@@ -270,8 +286,7 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
                     }
 #pragma unroll
                     for (int i = 0; i < ROWS; ++i) sa += av[i] * s[i];
-                    sa.x = reduce_rows<VQ>(sa.x); sa.y = reduce_rows<VQ>(sa.y);
-                    sa.z = reduce_rows<VQ>(sa.z); sa.w = reduce_rows<VQ>(sa.w);
+                    reduce_rows4<VQ>(sa);
                     if (ks == 0) *reinterpret_cast<float4_t*>(&sa_buf[t0 + tt][col0]) = sa;
 #pragma unroll
                     for (int i = 0; i < ROWS; ++i) s[i] = d[i] * s[i] + bv[i] * sa + kv[i] * v4;
@@ -315,14 +330,10 @@ void bwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
                     dv4 += kv[i] * Hd[i];
                     dsa4 += bv[i] * Hd[i];
                 }
-                dv4.x = reduce_rows<VQ>(dv4.x); dv4.y = reduce_rows<VQ>(dv4.y);
-                dv4.z = reduce_rows<VQ>(dv4.z); dv4.w = reduce_rows<VQ>(dv4.w);
-                dsa4.x = reduce_rows<VQ>(dsa4.x); dsa4.y = reduce_rows<VQ>(dsa4.y);
-                dsa4.z = reduce_rows<VQ>(dsa4.z); dsa4.w = reduce_rows<VQ>(dsa4.w);
-                if (ks == 0) {
-                    const float o4[4] = {dv4.x, dv4.y, dv4.z, dv4.w};
-                    Io<T>::store4(dv + base + (int64_t)(s0 + t0 + tt) * step + col0, o4);
-                }
+                const float dv1 = reduce_rows4_scattered<VQ>(dv4);     // row r of the wave: column col0 + r
+                reduce_rows4<VQ>(dsa4);
+                if ((lane & 15) < VQ)
+                    Io<T>::store1(dv + base + (int64_t)(s0 + t0 + tt) * step + col0 + (lane >> 4), dv1);
 #pragma unroll
                 for (int i = 0; i < ROWS; ++i) {
                     const float p_da = reduce_cols<VQ>(dot4(hp[i], dsa4));

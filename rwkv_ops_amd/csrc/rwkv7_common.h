@@ -100,6 +100,29 @@ __device__ __forceinline__ float sum_lane_groups_of_8(float x) {
     return __uint_as_float(r32[0]) + __uint_as_float(r32[1]);
 }
 
+// Four values at once over the four 16-lane rows of a wave (lanes l, l + 16, l + 32, l + 48).  A swap of two
+// DIFFERENT registers followed by one add halves two sums at a time: after v_permlane16_swap(a, b) the first
+// register holds rows (a0, b0, a2, b2) and the second (a1, b1, a3, b3), so their sum holds a0 + a1 in row 0 and
+// b0 + b1 in row 1; the same with c and d, then one v_permlane32_swap of the two sums and an add: row r of the
+// result is the total of value r.  Three swaps and three adds where value by value takes eight swaps, eight moves
+// and eight adds.
+__device__ __forceinline__ float sum4_over_rows_scattered(float a, float b, float c, float d) {
+    const auto s1 = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    const float ab = __uint_as_float(s1[0]) + __uint_as_float(s1[1]);
+    const auto s2 = __builtin_amdgcn_permlane16_swap(__float_as_uint(c), __float_as_uint(d), false, false);
+    const float cd = __uint_as_float(s2[0]) + __uint_as_float(s2[1]);
+    const auto s3 = __builtin_amdgcn_permlane32_swap(__float_as_uint(ab), __float_as_uint(cd), false, false);
+    return __uint_as_float(s3[0]) + __uint_as_float(s3[1]);
+}
+// ... and handed back to every row: rows (A, B, C, D) -> (A, B, A, B) and (C, D, C, D) -> A, B, C, D everywhere
+__device__ __forceinline__ void sum4_over_rows(float& a, float& b, float& c, float& d) {
+    const float t = sum4_over_rows_scattered(a, b, c, d);
+    const auto g1 = __builtin_amdgcn_permlane32_swap(__float_as_uint(t), __float_as_uint(t), false, false);
+    const auto g2 = __builtin_amdgcn_permlane16_swap(g1[0], g1[0], false, false);
+    const auto g3 = __builtin_amdgcn_permlane16_swap(g1[1], g1[1], false, false);
+    a = __uint_as_float(g2[0]); b = __uint_as_float(g2[1]); c = __uint_as_float(g3[0]); d = __uint_as_float(g3[1]);
+}
+
 // ---- N consecutive elements -> float --------------------------------------------
 template <typename T> struct Io;
 

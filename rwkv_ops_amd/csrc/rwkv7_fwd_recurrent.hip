@@ -22,12 +22,26 @@
 namespace rwkv7 {
 
 namespace {
-// sum over the lanes that share lane % VQ (VQ = 4: sixteen lanes, VQ = 8: eight), delivered to all of them
+// Sums over the lanes that share lane % VQ (VQ = 4: sixteen lanes, VQ = 8: eight).
+// the part of that sum inside a 16-lane row
 template <int VQ>
-__device__ __forceinline__ float reduce_row_groups(float x) {
+__device__ __forceinline__ float reduce_in_row(float x) {
     if constexpr (VQ == 4)
         x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x124, 0xf, 0xf, true));   // row_ror:4
-    return sum_lane_groups_of_8(x);              // row_ror:8, then the rows, then the halves
+    x += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), 0x128, 0xf, 0xf, true));       // row_ror:8
+    return x;
+}
+// the four components of v summed over the row groups, to all lanes (two registers per lane swap: rwkv7_common.h)
+template <int VQ>
+__device__ __forceinline__ void reduce_row_groups4(float4_t& v) {
+    float a = reduce_in_row<VQ>(v.x), b = reduce_in_row<VQ>(v.y), c = reduce_in_row<VQ>(v.z), d = reduce_in_row<VQ>(v.w);
+    sum4_over_rows(a, b, c, d);
+    v = float4_t{a, b, c, d};
+}
+// ... component r to the 16-lane row r of the wave only
+template <int VQ>
+__device__ __forceinline__ float reduce_row_groups4_scattered(const float4_t& v) {
+    return sum4_over_rows_scattered(reduce_in_row<VQ>(v.x), reduce_in_row<VQ>(v.y), reduce_in_row<VQ>(v.z), reduce_in_row<VQ>(v.w));
 }
 constexpr int REC_TB = 16;                       // tokens per staged block
 }  // namespace
@@ -163,8 +177,7 @@ void fwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
             if constexpr (!V6) {
 #pragma unroll
                 for (int i = 0; i < ROWS; ++i) sa += av[i] * s[i];
-                sa.x = reduce_row_groups<VQ>(sa.x); sa.y = reduce_row_groups<VQ>(sa.y);
-                sa.z = reduce_row_groups<VQ>(sa.z); sa.w = reduce_row_groups<VQ>(sa.w);
+                reduce_row_groups4<VQ>(sa);
             }
             if (!V6 && o == nullptr) {                  // the states only
 #pragma unroll
@@ -183,12 +196,9 @@ void fwd_recurrent_kernel(const T* __restrict__ r, const T* __restrict__ w, cons
                     acc += rv[i] * s[i];
                 }
             }
-            acc.x = reduce_row_groups<VQ>(acc.x); acc.y = reduce_row_groups<VQ>(acc.y);
-            acc.z = reduce_row_groups<VQ>(acc.z); acc.w = reduce_row_groups<VQ>(acc.w);
-            if (ks == 0 && o != nullptr) {
-                const float ov[4] = {acc.x, acc.y, acc.z, acc.w};
-                Io<T>::store4(o + base + (t0 + tt) * step + col0 + 4 * vq, ov);
-            }
+            const float o1 = reduce_row_groups4_scattered<VQ>(acc);    // row r of the wave: column col0 + 4 vq + r
+            if ((lane & 15) < VQ && o != nullptr)
+                Io<T>::store1(o + base + (t0 + tt) * step + col0 + 4 * vq + (lane >> 4), o1);
         }
     }
     if (ht != nullptr) {
