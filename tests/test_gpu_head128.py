@@ -218,3 +218,26 @@ def test_gradients_with_many_heads(device, T):
             assert rel_l2(g_, r_[:rows]) < 1e-4, (rows, name)
     for a_, b_ in zip(got[B], got[3]):
         assert rel_l2(a_[:3], b_) < 2e-6
+
+
+def test_gradients_at_the_benchmark_shape(device):
+    """B = 8, T = 1024, H = 16, bf16 (bench.py's head128.backward: 128 (batch, head) pairs, so the split form on all
+    256 CUs): four pairs, the corners of the batch among them, against float32 autograd through the oracle on the
+    same rounded inputs (heads and batch rows are independent, so the oracle runs on the slices)."""
+    B, T, H = 8, 1024, 16
+    xs = make_inputs(B, T, H, N, seed=9600, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(9601)
+    dO = torch.randn(B, T, H, N, generator=g).to(torch.bfloat16)
+    dS = 0.1 * torch.randn(B, H, N, N, generator=g)
+    leaves = [x.to(device).requires_grad_(True) for x in xs]
+    o, s = rwkv_ops_amd.generalized_delta_rule(*leaves[:6], initial_state=leaves[6])
+    loss = (o.float() * dO.to(device).float()).sum() + (s * dS.to(device)).sum()
+    got = [t.cpu() for t in torch.autograd.grad(loss, leaves)]
+    names = ["dr", "dw", "dk", "dv", "da", "db", "dh0"]
+    for b, h in ((0, 0), (B - 1, H - 1), (0, H - 1), (3, 7)):
+        one = [x[b:b + 1, :, h:h + 1].contiguous() for x in xs[:6]] + [xs[6][b:b + 1, h:h + 1].contiguous()]
+        ref = orc.gradients(*one[:6], one[6], dO[b:b + 1, :, h:h + 1].contiguous(), dS[b:b + 1, h:h + 1].contiguous())
+        for j, name in enumerate(names):
+            mine = got[j][b:b + 1, h:h + 1] if name == "dh0" else got[j][b:b + 1, :, h:h + 1]
+            e = rel_l2(mine, ref[j])
+            assert e < (1e-4 if name == "dh0" else 4e-3), (b, h, name, e)
