@@ -357,8 +357,7 @@ void chunk_bwd_body(int n, int lane, const ChunkInputs& in, ChunkInputs& next, i
 #pragma unroll
         for (int e = 0; e < 8; ++e) { gl[e] += pre[e]; xmax = fmaxf(xmax, fmaxf(-gsum[e], -gother[e])); }
     }
-    xmax = fmaxf(xmax, __shfl_xor(xmax, 16, 64));
-    xmax = fmaxf(xmax, __shfl_xor(xmax, 32, 64));
+    xmax = max_over_rows(xmax);
     const int npass = (int)(xmax * (1.f / BUCKET2)) + 1;       // uniform over the workgroup
     if constexpr (!GENERAL) {
         if (npass > 1) {

@@ -508,8 +508,7 @@ void chunk16_f32_bwd_grad_kernel(const float* __restrict__ r_, const float* __re
     float4_t hd4;
     {
         float hd = (hdp[0] + hdp[1]) + (hdp[2] + hdp[3]);
-        hd += __shfl_xor(hd, 16, 64);
-        hd += __shfl_xor(hd, 32, 64);
+        hd = sum_over_rows(hd);
         float* hdl = reinterpret_cast<float*>(smem + G_HD + w * 64);
         if (g == 0) hdl[x] = hd;
         hd4 = *reinterpret_cast<const float4_t*>(hdl + 4 * g);

@@ -100,6 +100,21 @@ __device__ __forceinline__ float sum_lane_groups_of_8(float x) {
     return __uint_as_float(r32[0]) + __uint_as_float(r32[1]);
 }
 
+// Maximum / sum of x over the four 16-lane rows of a wave (lanes l, l ^ 16, l ^ 32, l ^ 48), to all of them: the two
+// swaps instead of two __shfl_xor, each of which is a trip through the LDS crossbar (72 cycles against 24).
+__device__ __forceinline__ float max_over_rows(float x) {
+    const auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = fmaxf(__uint_as_float(r16[0]), __uint_as_float(r16[1]));
+    const auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r32[0]), __uint_as_float(r32[1]));
+}
+__device__ __forceinline__ float sum_over_rows(float x) {
+    const auto r16 = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    x = __uint_as_float(r16[0]) + __uint_as_float(r16[1]);
+    const auto r32 = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r32[0]) + __uint_as_float(r32[1]);
+}
+
 // Four values at once over the four 16-lane rows of a wave (lanes l, l + 16, l + 32, l + 48).  A swap of two
 // DIFFERENT registers followed by one add halves two sums at a time: after v_permlane16_swap(a, b) the first
 // register holds rows (a0, b0, a2, b2) and the second (a1, b1, a3, b3), so their sum holds a0 + a1 in row 0 and

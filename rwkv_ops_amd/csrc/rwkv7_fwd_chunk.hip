@@ -267,8 +267,7 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
     float xmax = 0.f;
 #pragma unroll
     for (int e = 0; e < 16; ++e) xmax = fmaxf(xmax, -gsum[e]);
-    xmax = fmaxf(xmax, __shfl_xor(xmax, 16, 64));
-    xmax = fmaxf(xmax, __shfl_xor(xmax, 32, 64));
+    xmax = max_over_rows(xmax);
     const int npass = (int)(xmax * (1.f / BUCKET)) + 1;
 
     if (w == 0 && x == 0) {            // decay of the whole chunk per key channel
@@ -296,8 +295,7 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         unpack8(load_frag_global(fa.u + hi * HEAD + 32 + 8 * g, true), uf + 8);
 #pragma unroll
         for (int e = 0; e < 16; ++e) bonus = fmaf(rf[e] * uf[e], kf[e], bonus);
-        bonus += __shfl_xor(bonus, 16, 64);
-        bonus += __shfl_xor(bonus, 32, 64);
+        bonus = sum_over_rows(bonus);
     }
     bf16x8_t QG[2], AG[2], KG[2], BG[2];
     auto scale_operands = [&](auto single_bucket) {

@@ -209,8 +209,7 @@ void chunk128_fwd_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restrict
             float xmax = 0.f;
 #pragma unroll
             for (int e = 0; e < 16; ++e) xmax = fmaxf(xmax, -gsum[e]);
-            xmax = fmaxf(xmax, __shfl_xor(xmax, 16, 64));
-            xmax = fmaxf(xmax, __shfl_xor(xmax, 32, 64));
+            xmax = max_over_rows(xmax);
             if (lane == 0) reinterpret_cast<float*>(smem + OFF_XM)[wv] = xmax;
             if (w == 0 && x == 0) {        // decay of the whole chunk per key channel
                 float* eg = reinterpret_cast<float*>(smem + OFF_EG);
@@ -268,8 +267,7 @@ void chunk128_fwd_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restrict
                     sa4 += a4 * h[ct];
                 }
                 float sa = (sa4.x + sa4.y) + (sa4.z + sa4.w);
-                sa += __shfl_xor(sa, 16, 64);
-                sa += __shfl_xor(sa, 32, 64);
+                sa = sum_over_rows(sa);
                 float4_t o4 = zero4;
                 const float vf = (float)vv;
 #pragma unroll
@@ -283,8 +281,7 @@ void chunk128_fwd_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restrict
                     o4 += r4 * h[ct];
                 }
                 float ov = (o4.x + o4.y) + (o4.z + o4.w);
-                ov += __shfl_xor(ov, 16, 64);
-                ov += __shfl_xor(ov, 32, 64);
+                ov = sum_over_rows(ov);
                 if (g == 0) o_[((sp.tok0 + c * CH + tt) * H + hi) * N + 16 * wv + x] = (bf16_t)ov;
             }
             __syncthreads();               // the next chunk rewrites the tiles

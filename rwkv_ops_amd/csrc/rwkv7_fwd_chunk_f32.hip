@@ -291,8 +291,7 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
 #pragma unroll
                 for (int ct = 0; ct < 4; ++ct) sa4 += tile4(smem, F_AG, tt, 16 * ct + 4 * g) * h[ct];
                 float sa = (sa4[0] + sa4[1]) + (sa4[2] + sa4[3]);
-                sa += __shfl_xor(sa, 16, 64);
-                sa += __shfl_xor(sa, 32, 64);
+                sa = sum_over_rows(sa);
                 float4_t o4 = zero4;
 #pragma unroll
                 for (int ct = 0; ct < 4; ++ct) {
@@ -301,8 +300,7 @@ void chunk16_f32_fwd_kernel(const float* __restrict__ r_, const float* __restric
                     o4 += tile4(smem, F_RAW_R, tt, col) * h[ct];
                 }
                 float ov = (o4[0] + o4[1]) + (o4[2] + o4[3]);
-                ov += __shfl_xor(ov, 16, 64);
-                ov += __shfl_xor(ov, 32, 64);
+                ov = sum_over_rows(ov);
                 if (g == 0 && o_ != nullptr) o_[((sp.tok0 + c * C16 + tt) * H + hi) * NH + 16 * w + x] = ov;
             }
             __syncthreads();
