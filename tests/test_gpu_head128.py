@@ -241,3 +241,38 @@ def test_gradients_at_the_benchmark_shape(device):
             mine = got[j][b:b + 1, h:h + 1] if name == "dh0" else got[j][b:b + 1, :, h:h + 1]
             e = rel_l2(mine, ref[j])
             assert e < (1e-4 if name == "dh0" else 4e-3), (b, h, name, e)
+
+
+@pytest.mark.parametrize("B,H", [(3, 2), (50, 4)])
+def test_float32_forward_variants(device, B, H):
+    """float32 tensors at head size 128 take the recurrent forward: two workgroups per (batch, head) up to 192 pairs
+    (6 here), one beyond (200).  No initial state, a shared one, a state map, packed sequences with an empty one and
+    rows behind the last: against the oracle, 1e-4."""
+    from oracle import native_c
+    T = 45
+    xs = make_inputs(B, T, H, N, seed=9700, dtype=torch.float32)
+    d = [x.to(device) for x in xs]
+    with torch.no_grad():
+        o, s = rwkv_ops_amd.generalized_delta_rule(*d[:6])
+        o_ref, s_ref = native_c.run(*xs[:6], None)
+        assert rel_l2(o, o_ref) < 1e-4 and rel_l2(s, s_ref) < 1e-4
+        o, s = rwkv_ops_amd.generalized_delta_rule(*d[:6], initial_state=d[6][:1])
+        o_ref, s_ref = native_c.run(*xs[:6], xs[6][:1])
+        assert rel_l2(o, o_ref) < 1e-4 and rel_l2(s, s_ref) < 1e-4
+        smap = [(2 * i + 1) % B for i in range(B)]
+        o, s = rwkv_ops_amd.generalized_delta_rule(*d[:6], initial_state=d[6], state_map=smap)
+        o_ref, s_ref = native_c.run(*xs[:6], xs[6][smap])
+        assert rel_l2(o, o_ref) < 1e-4 and rel_l2(s, s_ref) < 1e-4
+        # the first two batch rows as one packed row: lengths 45, 0, 30, 15, and 10 rows behind the last sequence
+        row = [torch.cat([x[0], x[1], x[2][:10]], 0)[None].contiguous() for x in d[:6]]
+        cu = [0, 45, 45, 75, 90]
+        h4 = d[6][[0, 1, 2, 0]].contiguous()
+        o, s = rwkv_ops_amd.generalized_delta_rule(*row, initial_state=h4, cu_seqlens=cu)
+        for i in range(4):
+            a_, b_ = cu[i], cu[i + 1]
+            if a_ == b_:
+                assert torch.equal(s[i], h4[i])
+                continue
+            o_ref, s_ref = native_c.run(*[x[:, a_:b_].cpu() for x in row], h4[i:i + 1].cpu())
+            assert rel_l2(o[:, a_:b_], o_ref) < 1e-4 and rel_l2(s[i:i + 1], s_ref) < 1e-4, i
+        assert float(o[:, 90:].abs().max()) == 0.0
