@@ -157,10 +157,9 @@ int rwkv7_fwd(const void* r, const void* w, const void* k, const void* v, const 
 
 /* ---- the forward for callers that may not allocate -------------------------------------------- */
 namespace {
-// The one-kernel forward's workspace (hand-off counters, status record, two state slots per (batch, head))
+// The one-kernel forward's workspace (status record, two state slots per (batch, head) and their carriers)
 // for RWKV7_NOALLOC_MAX_BH sequences, held by every GPU the library is loaded on until the process ends.
-constexpr size_t SCRATCH_BYTES =
-    (((size_t)RWKV7_NOALLOC_MAX_BH * 32 + 16 + 255) / 256) * 256 + 2 * (size_t)RWKV7_NOALLOC_MAX_BH * 4096 * 4;
+constexpr size_t SCRATCH_BYTES = rwkv7::fwd_fused_bytes(RWKV7_NOALLOC_MAX_BH);
 static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
 // The array's name is a host-side stand-in; its device address differs per GPU and is looked up once per
 // device (with that device current) and kept here.

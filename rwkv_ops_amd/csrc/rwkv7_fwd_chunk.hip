@@ -88,26 +88,71 @@ __device__ __forceinline__ bf16x8_t load_frag_global(const bf16_t* p, bool valid
 
 // Device-scope ("sc1") 16-byte accesses for the state hand-off of the fused kernel: four 16-byte
 // pieces 1 KiB apart per lane (the four key tiles of one value tile of a state image).  They bypass
-// the per-XCD L2, so a workgroup on any XCD sees what another one wrote once the writer's
-// s_waitcnt vmcnt(0) has returned.  Vector memory instructions only.
-__device__ __forceinline__ void state_store_agent(float* p, const float4_t (&h)[4]) {
+// the per-XCD L2, so a workgroup on any XCD sees what another one wrote.  Vector memory instructions only.
+// (Keeping the image in the L2 of the XCD that both workgroups of a head run on was measured: a load that
+// passes the CU's own cache but stops at L2 does not exist below device scope, and invalidating the CU's
+// cache per poll costs more than the trip to memory.)
+__device__ __forceinline__ void state_store(float* p, uint32_t* pc, const float4_t (&h)[4], uint32_t car) {
     asm volatile("global_store_dwordx4 %0, %1, off sc1\n\t"
                  "global_store_dwordx4 %0, %2, off offset:1024 sc1\n\t"
                  "global_store_dwordx4 %0, %3, off offset:2048 sc1\n\t"
-                 "global_store_dwordx4 %0, %4, off offset:3072 sc1"
-                 :: "v"(p), "v"(h[0]), "v"(h[1]), "v"(h[2]), "v"(h[3]) : "memory");
+                 "global_store_dwordx4 %0, %4, off offset:3072 sc1\n\t"
+                 "global_store_dword %5, %6, off sc1"
+                 :: "v"(p), "v"(h[0]), "v"(h[1]), "v"(h[2]), "v"(h[3]), "v"(pc), "v"(car) : "memory");
 }
 // Issue and arrival are separate so that other work can sit between them; the second statement
 // names the registers again, which keeps every use of them behind the wait.
-__device__ __forceinline__ void state_load_agent_issue(const float* p, float4_t (&h)[4]) {
-    asm volatile("global_load_dwordx4 %0, %4, off sc1\n\t"
-                 "global_load_dwordx4 %1, %4, off offset:1024 sc1\n\t"
-                 "global_load_dwordx4 %2, %4, off offset:2048 sc1\n\t"
-                 "global_load_dwordx4 %3, %4, off offset:3072 sc1"
-                 : "=&v"(h[0]), "=&v"(h[1]), "=&v"(h[2]), "=&v"(h[3]) : "v"(p) : "memory");
+__device__ __forceinline__ void state_load_issue(const float* p, const uint32_t* pc, float4_t (&h)[4], uint32_t& car) {
+    asm volatile("global_load_dwordx4 %0, %5, off sc1\n\t"
+                 "global_load_dwordx4 %1, %5, off offset:1024 sc1\n\t"
+                 "global_load_dwordx4 %2, %5, off offset:2048 sc1\n\t"
+                 "global_load_dwordx4 %3, %5, off offset:3072 sc1\n\t"
+                 "global_load_dword %4, %6, off sc1"
+                 : "=&v"(h[0]), "=&v"(h[1]), "=&v"(h[2]), "=&v"(h[3]), "=&v"(car) : "v"(p), "v"(pc) : "memory");
 }
-__device__ __forceinline__ void state_load_agent_wait(float4_t (&h)[4]) {
-    asm volatile("s_waitcnt vmcnt(0)" : "+v"(h[0]), "+v"(h[1]), "+v"(h[2]), "+v"(h[3]) :: "memory");
+__device__ __forceinline__ void state_load_wait(float4_t (&h)[4], uint32_t& car) {
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(h[0]), "+v"(h[1]), "+v"(h[2]), "+v"(h[3]), "+v"(car) :: "memory");
+}
+
+// The hand-off carries its own "ready" marks, so that a reader needs no separate counter and no second
+// trip to memory: it loads the image and looks at the marks.  An image is, per lane, four 16-byte words
+// (sixteen floats of the state) and one 4-byte "carrier".  In the first and the last float of every 16-byte
+// word a 3-bit field (bits 8+3j .. 10+3j for the j-th such float, j = 0..7) is replaced by a mark; the bits
+// that stood there travel in the same field of the carrier, whose low 8 bits are its own mark, and the reader
+// puts them back: the state crosses the hand-off bit for bit.  The marks of chunk c are the fields of
+//     E(c) = S(1 + (c / 2) mod 7) ^ tag32,   S(v) = v in every 3-bit field and v | v << 3 in the low byte,
+// so the fields of two images that follow each other in a slot differ (as do those seven uses apart), and a
+// cleared slot holds S(0) ^ tag32 = tag32 in every 4-byte piece, which is no chunk's mark in any field.  An
+// image half arrived still shows an old field somewhere: two fields per 16-byte word catch a word torn at
+// 8 bytes or coarser (the memory system moves 32 bytes or more at a time).
+__device__ __forceinline__ uint32_t handoff_marks(unsigned long long tag, int c) {
+    const uint32_t v = 1u + (uint32_t)(c >> 1) % 7u;
+    return (v * 0x24924900u | v * 9u) ^ (uint32_t)tag;
+}
+__device__ __forceinline__ uint32_t bfi(uint32_t mask, uint32_t a, uint32_t b) { return (a & mask) | (b & ~mask); }
+// marks into the image, the bits they replace into the carrier (returned)
+__device__ __forceinline__ uint32_t handoff_mark(float4_t (&h)[4], uint32_t marks) {
+    uint32_t car = marks;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const uint32_t m = 7u << (8 + 3 * j), x = __float_as_uint(h[j >> 1][(j & 1) * 3]);
+        car = bfi(m, x, car);
+        h[j >> 1][(j & 1) * 3] = __uint_as_float(bfi(m, marks, x));
+    }
+    return car;
+}
+// true when this lane's part of the image and its carrier show the marks
+__device__ __forceinline__ bool handoff_marked(const float4_t (&h)[4], uint32_t car, uint32_t marks) {
+    uint32_t seen = car;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) seen = bfi(7u << (8 + 3 * j), __float_as_uint(h[j >> 1][(j & 1) * 3]), seen);
+    return seen == marks;
+}
+__device__ __forceinline__ void handoff_restore(float4_t (&h)[4], uint32_t car) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        h[j >> 1][(j & 1) * 3] = __uint_as_float(bfi(7u << (8 + 3 * j), car, __float_as_uint(h[j >> 1][(j & 1) * 3])));
+    }
 }
 
 }  // namespace
@@ -144,8 +189,8 @@ struct FusedArgs {
     bf16_t* o;
     float* ht;                 // nullable
     float* hbuf;               // [2][B*H][4 value tiles][4 key tiles][64 lanes][4] float hand-off slots
-    unsigned long long* cnt;   // [B*H][4] tag + chunks completed per (head, value tile)
-    unsigned long long tag;    // this launch's random 64-bit tag: the counters need no clearing (see launch_fwd_fused)
+    uint32_t* hcar;            // [2][B*H][4 value tiles][64 lanes] the slots' carriers (see handoff_marks)
+    unsigned long long tag;    // this launch's random 64-bit tag: the slots need no clearing (see launch_fwd_fused)
     unsigned long long* status; // nullable: [0] = give-up flag (== tag: a hand-off wait timed out), [1] = tag of the launch
 };
 
@@ -621,7 +666,14 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         // issued before the exchange below and collected after it.
         float4_t h[4];
         const int slot_in = (c - 1) & 1, slot_out = c & 1;
-        bool ok = true;
+        float* const hin = fa.hbuf + ((int64_t)slot_in * BH + bh) * 4096 + (w * 4 * 64 + lane) * 4;
+        float* const hout = fa.hbuf + ((int64_t)slot_out * BH + bh) * 4096 + (w * 4 * 64 + lane) * 4;
+        uint32_t* const cin = fa.hcar + ((int64_t)slot_in * BH + bh) * 256 + w * 64 + lane;
+        uint32_t* const cout = fa.hcar + ((int64_t)slot_out * BH + bh) * 256 + w * 64 + lane;
+        const float cleared_f = __uint_as_float((uint32_t)fa.tag);
+        const float4_t cleared4 = {cleared_f, cleared_f, cleared_f, cleared_f};
+        const float4_t cleared[4] = {cleared4, cleared4, cleared4, cleared4};
+        uint32_t car = 0;
         if (c == 0) {
             if (fa.h0 != nullptr) {
                 const float* src = fa.h0 + state_row(fa.h0_map, fa.n_state, bi) * fa.h0_batch_stride + (int64_t)hi * STATE + 16 * w + x;
@@ -633,19 +685,43 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
 #pragma unroll
                 for (int ct = 0; ct < 4; ++ct) h[ct] = zero4;
             }
-        } else {
-            unsigned long long* cnt = fa.cnt + bh * 4 + w;
-            if (lane == 0) {
-                // The previous chunk's wave w publishes exactly tag + c.  Bounded wait: after WAIT_LIMIT_TICKS of
-                // the constant-rate clock without progress (or as soon as any other wave has given up) the wave
-                // stops waiting and poisons its outputs, so the grid always drains.  The clock and the shared
-                // flag are looked at once per 1024 polls.
-                const unsigned long long want = fa.tag + (unsigned long long)c;
+            if (NT > 1) {
+                // The first chunk of a sequence clears both slots of its head (this wave: its value tile), so that
+                // whatever the workspace held reads "not yet"; its own image follows after a wait for these stores.
+                state_store(hout, cout, cleared, (uint32_t)fa.tag);
+                state_store(hin, cin, cleared, (uint32_t)fa.tag);
+            }
+        }
+        // Wave w now plays value tile w of the scan: it needs ALL of Qt and Pp (the other waves hold the
+        // other halves), so the halves go through LDS into the tiles that the chains no longer read.
+        __syncthreads();
+        if (c != 0) state_load_issue(hin, cin, h, car);      // a first look at the slot, collected behind the exchange below
+        bf16_t* fq = reinterpret_cast<bf16_t*>(smem + OFF_AG);       // [4 tiles][2 k-steps][2 halves][64][4]
+        bf16_t* fp = reinterpret_cast<bf16_t*>(smem + OFF_V);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            *reinterpret_cast<bf16x4_t*>(fq + ((m * 4 + w) * 64 + lane) * 4) = qth[m];
+            *reinterpret_cast<bf16x4_t*>(fp + ((m * 4 + w) * 64 + lane) * 4) = pph[m];
+        }
+        __syncthreads();
+        if (c != 0) {
+            // The previous chunk's workgroup (lower block index, hence dispatched earlier) publishes value tile w
+            // with the marks of chunk c - 1.  Bounded wait: after WAIT_LIMIT_TICKS of the constant-rate clock
+            // without the image (or as soon as any other wave has given up) the wave stops waiting and poisons
+            // its outputs, so the grid always drains.  The clock and the shared flag are looked at once per 256
+            // polls (a poll is a trip to L2 or to memory).
+            const uint32_t want = handoff_marks(fa.tag, c - 1);
+            state_load_wait(h, car);
+            bool ok = true;
+            if (!__all(handoff_marked(h, car, want))) {
                 unsigned spins = 0;
                 unsigned long long t0 = 0;
-                while (__hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want) {
+                for (;;) {
                     __builtin_amdgcn_s_sleep(1);
-                    if ((++spins & 1023u) == 0) {
+                    state_load_issue(hin, cin, h, car);
+                    state_load_wait(h, car);
+                    if (__all(handoff_marked(h, car, want))) break;
+                    if ((++spins & 255u) == 0) {
                         const unsigned long long now = wall_clock64();
                         if (t0 == 0) t0 = now;
                         if (now - t0 > WAIT_LIMIT_TICKS ||
@@ -656,31 +732,16 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
                         }
                     }
                 }
-                // The last chunk is this counter's last reader: it takes the value away, so that a replay of
-                // the same launch (a captured graph repeats the tag) does not find it there before its time.
-                if (c + 1 == NT)
-                    __hip_atomic_store(cnt, fa.tag - 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
-            ok = __shfl((int)ok, 0, 64) != 0;
-            state_load_agent_issue(fa.hbuf + ((int64_t)slot_in * BH + bh) * 4096 + (w * 4 * 64 + lane) * 4, h);
-        }
-        // Wave w now plays value tile w of the scan: it needs ALL of Qt and Pp (the other waves hold the
-        // other halves), so the halves go through LDS into the tiles that the chains no longer read.
-        __syncthreads();
-        bf16_t* fq = reinterpret_cast<bf16_t*>(smem + OFF_AG);       // [4 tiles][2 k-steps][2 halves][64][4]
-        bf16_t* fp = reinterpret_cast<bf16_t*>(smem + OFF_V);
-#pragma unroll
-        for (int m = 0; m < 4; ++m) {
-            *reinterpret_cast<bf16x4_t*>(fq + ((m * 4 + w) * 64 + lane) * 4) = qth[m];
-            *reinterpret_cast<bf16x4_t*>(fp + ((m * 4 + w) * 64 + lane) * 4) = pph[m];
-        }
-        __syncthreads();
-        if (c != 0) {
-            state_load_agent_wait(h);
-            if (!ok) {
+            if (ok) {
+                handoff_restore(h, car);
+            } else {
 #pragma unroll
                 for (int ct = 0; ct < 4; ++ct) h[ct] = float4_t{__builtin_nanf(""), __builtin_nanf(""), __builtin_nanf(""), __builtin_nanf("")};
             }
+            // No later chunk of this launch writes the slot just read: clear it, so that a replay of the same
+            // launch (a captured graph repeats the tag) cannot take this image for its own.
+            if (c + 2 >= NT) state_store(hin, cin, cleared, (uint32_t)fa.tag);
         }
         bf16x8_t bhi[2], blo[2];
         split_sigma(h[0], h[1], bhi[0], blo[0]);
@@ -710,7 +771,10 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         // send the new state on its way first (the next chunk needs it); the counter that announces it
         // is bumped after the output products below, which run while the stores are in flight
         if (c + 1 < NT) {
-            state_store_agent(fa.hbuf + ((int64_t)slot_out * BH + bh) * 4096 + (w * 4 * 64 + lane) * 4, hn);
+            if (c == 0) __builtin_amdgcn_s_waitcnt(0);       // the clearing stores above have been acknowledged
+            float4_t hm[4] = {hn[0], hn[1], hn[2], hn[3]};
+            const uint32_t carried = handoff_mark(hm, handoff_marks(fa.tag, c));
+            state_store(hout, cout, hm, carried);
         } else if (fa.ht != nullptr) {
             float* dst = fa.ht + (int64_t)bh * STATE + 16 * w + x;
 #pragma unroll
@@ -733,12 +797,6 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
                 acc = mfma_bf16(a8, blo[s], acc);
             }
             *reinterpret_cast<bf16x4_t*>(smem + OFF_QG + ((16 * w + x) * LDQ + 16 * it + 4 * g) * 2) = pack4(acc);
-        }
-        if (c + 1 < NT) {
-            __builtin_amdgcn_s_waitcnt(0);                   // every state store of this wave has been acknowledged
-            if (lane == 0)
-                __hip_atomic_store(fa.cnt + bh * 4 + w, fa.tag + (unsigned long long)(c + 1), __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
         }
         __syncthreads();
 #pragma unroll
@@ -1267,13 +1325,11 @@ hipError_t launch_fwd_chunk(const SeqArgs& p, void* ws, hipStream_t stream) {
 }
 
 size_t fwd_fused_status_offset(int B, int T, int H, bool varlen) {
-    return (size_t)B * H * 32 + (varlen ? chunk_items_bytes(B, T) : 0);
+    return varlen ? chunk_items_bytes(B, T) : 0;
 }
 
 size_t fwd_fused_workspace_bytes(int B, int T, int H, bool varlen) {
-    const size_t bh = (size_t)B * H;
-    // 8-byte counters (one per head and value tile), a 16-byte status record, then two state slots per head
-    return ((bh * 32 + 16 + 255) / 256) * 256 + 2 * bh * 4096 * 4 + (varlen ? chunk_items_bytes(B, T) : 0);
+    return fwd_fused_bytes((size_t)B * H) + (varlen ? chunk_items_bytes(B, T) : 0);
 }
 
 hipError_t launch_fwd_fused(const SeqArgs& p, void* ws, hipStream_t stream) {
@@ -1288,14 +1344,14 @@ hipError_t launch_fwd_fused(const SeqArgs& p, void* ws, hipStream_t stream) {
     FusedArgs fa{};
     fa.h0 = p.h0; fa.h0_batch_stride = p.h0_batch_stride; fa.h0_map = p.h0_map; fa.n_state = p.n_state;
     fa.o = (bf16_t*)p.o; fa.ht = p.ht;
-    fa.cnt = reinterpret_cast<unsigned long long*>(base);
-    fa.hbuf = reinterpret_cast<float*>(base + (((size_t)BH * 32 + 16 + 255) / 256) * 256);
-    fa.status = fa.cnt + (size_t)BH * 4;
-    // The hand-off counters are compared for EQUALITY with tag + chunk index, so whatever the workspace
-    // holds on entry (an earlier launch's counters, or anything else) reads as "not there yet" unless it
-    // equals one specific 64-bit value, and no clearing launch is needed in front of the kernel.  A
-    // captured graph replays the same tag; the kernel's last chunk removes the one value a replay could
-    // mistake (see there).
+    // the status record (padded to 256 bytes), two state slots per head, then the slots' carriers
+    fa.status = reinterpret_cast<unsigned long long*>(base);
+    fa.hbuf = reinterpret_cast<float*>(base + 256);
+    fa.hcar = reinterpret_cast<uint32_t*>(base + 256 + 2 * (size_t)BH * 4096 * 4);
+    // A slot's content is judged by marks that depend on this launch's tag (handoff_marks), and the first chunk
+    // of every sequence clears its head's slots, so whatever the workspace holds on entry reads as "not there
+    // yet" and no clearing launch is needed in front of the kernel.  A captured graph replays the same tag; the
+    // readers of a head's last images clear them (see there).
     fa.tag = next_launch_tag();
     fa.u = static_cast<const bf16_t*>(p.u6);
     return p.u6 ? launch_summary_kernel<MODE_FUSED, true>(p, nchunks, nullptr, nullptr, nullptr, nullptr, nullptr, L, fa, stream)

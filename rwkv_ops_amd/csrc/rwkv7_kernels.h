@@ -37,6 +37,9 @@ hipError_t launch_fwd_chunk(const SeqArgs& p, void* ws, hipStream_t stream);
 // the same forward as ONE kernel: each chunk's workgroup applies its summary to the state it receives
 // from the previous chunk's workgroup and hands the new state on (ws: fwd_fused_workspace_bytes)
 size_t fwd_fused_workspace_bytes(int B, int T, int H, bool varlen = false);
+// ... of which, for bh (batch, head) sequences: the status record padded to 256 bytes, two float32 state slots
+// per sequence and head and the slots' 1 KiB carriers
+constexpr size_t fwd_fused_bytes(size_t bh) { return 256 + 2 * bh * (4096 * 4 + 1024); }
 // Byte offset, within the workspace of either form, of the launch's 16-byte status record (two 64-bit
 // words): [1] = the launch's tag (never 0), [0] = that tag if a hand-off wait of the one-kernel form timed
 // out and the outputs were poisoned, anything else otherwise.
