@@ -44,32 +44,64 @@ constexpr int CH = 64;                 // tokens per chunk
 // computed), so that each later exponential is a bare v_exp_f32.
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float BUCKET = 64.f * LOG2E; // exponent range of one pass (e^64), in base-2 units
-constexpr float G_MIN = -87.f * LOG2E; // per-step log-decay clamp (e^-87 is below FLT_MIN), in base-2 units
+constexpr float X_STEP_MAX = 87.f * LOG2E;     // per-step clamp of -log2 decay (e^-87 is below FLT_MIN)
+constexpr float LOG2_LOG2E = 0.5287663729448977f;   // log2(log2 e)
 __device__ __forceinline__ float ex2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// LDS map of chunk_summary_kernel (bytes)
-constexpr int OFF_KT = 0;              // k~ A-fragments [4 J][2 s][64 lanes][8] bf16
+// LDS map of chunk_summary_kernel (bytes).  Regions are reused along the phases of a chunk ("B1" ... name
+// the workgroup barriers in the kernel); 50.6 KiB in all, so that three workgroups share a CU's 160 KiB.
+constexpr int OFF_KT = 0;              // k~ A-fragments [4 J][2 s][64 lanes][8] bf16                      B1 .. end
 constexpr int OFF_BT = 8192;           // b~
-constexpr int OFF_AAB = 16384;         // 10 lower-triangular 16x16 bf16 blocks of Aab, row-major [i][j] (512 B each)
-constexpr int OFF_DI = 26624;          // 4 inverted diagonal blocks, bf16, row-major (512 B each)
-constexpr int OFF_KG = 0;              // (after the inverse) kg row-major [64][LDT]
-constexpr int OFF_BG = 10240;          // bg
-constexpr int OFF_QG = 30720;          // qg row-major [64][LDQ]
-constexpr int OFF_AG = 39936;          // ag row-major [64][LDT]
-constexpr int OFF_V = 50176;           // v
-constexpr int OFF_AQK = 60416;         // 6 sigma fragments of Aqk [i][j]
-constexpr int OFF_AQB = 66560;
-constexpr int OFF_AAK = 72704;
-constexpr int OFF_TOT = 78848;         // float [4 sub-blocks][64 channels]
-constexpr int OFF_EG = 79872;          // float [64]: e^G per key channel (fused kernel)
-constexpr int LDS_BYTES = 80128;
-constexpr int LDT = 80;                // row stride (elements) of tiles read with the transposing load
-constexpr int LDQ = 72;
+constexpr int OFF_KG = 0;              // several buckets only: the kg, bg tiles, once k~, b~ are done with
+constexpr int OFF_BG = 8192;
+constexpr int OFF_V = 16384;           // v tile                                                          B1 .. Bx
+constexpr int OFF_AAK = 16384;         //   then the 6 sigma fragments of Aak [i][j]                       Bx .. B3
+constexpr int OFF_QG = 16384;          //   then the qg tile                                               B3 .. Bf1
+constexpr int OFF_FP = 16384;          //   then (fused) the exchanged halves of Pp
+constexpr int OFF_AG = 24576;          // ag tile                                                         B1 .. B4
+constexpr int OFF_DO = 24576;          //   then (backward) the dO tile
+constexpr int OFF_FQ = 24576;          //   then (fused) the exchanged halves of Qt
+constexpr int OFF_AQK = 32768;         // 6 sigma fragments of Aqk [i][j]                                  Bx .. Bf1
+constexpr int OFF_AQB = 38912;
+constexpr int OFF_OT = 32768;          //   then (fused) the O tile, transposed
+constexpr int OFF_AAB = 45056;         // the 6 blocks of Aab below the diagonal, 16x16 bf16 row-major [i][j] (512 B each)
+constexpr int OFF_DI = 48128;          // 4 inverted diagonal blocks, bf16, row-major (512 B each)
+constexpr int OFF_EG = 50176;          // float [64]: e^G per key channel
+constexpr int OFF_TOT = 50432;         // float [4 waves][64 channels]: each wave's decay totals (kept to the end)
+constexpr int OFF_TMAX = 51456;        // float [4]: the largest total of each wave
+constexpr int LDS_BYTES = 51712;
+constexpr int LDT = 80;                // row stride (elements) of the scan kernels' O tiles
 
 // fragment index of the lower-triangular [i][j] matrices: (i tile, k-step) with s <= it / 2
 __device__ __forceinline__ constexpr int fidx(int it, int s) { return it < 2 ? it : 2 + (it - 2) * 2 + s; }
-// index of the float block (I, J), J <= I
-__device__ __forceinline__ constexpr int bidx(int I, int J) { return I * (I + 1) / 2 + J; }
+// index of the block (I, J) below the diagonal, J < I
+__device__ __forceinline__ constexpr int lidx(int I, int J) { return I * (I - 1) / 2 + J; }
+
+// The 64 x 64 bf16 tiles of the summary kernel are 8 KiB, rows of 128 bytes with the eight 16-byte pieces of
+// row r stored at piece ^ (r & 7): a 16-byte row access, an 8-byte piece of a row and the transposing read
+// (four consecutive rows per group of 16 lanes) all spread over the banks as they do with padded rows.
+__device__ __forceinline__ int tile_at(int row, int col) {          // col a multiple of 4
+    return row * 128 + ((((col >> 3) ^ row) & 7) << 4) + ((col & 7) << 1);
+}
+// "sigma" fragment of the TRANSPOSE of such a tile: lane (x, g) receives column 16 ct + x of rows
+// 32 s + 4 g + (0..3) and 32 s + 16 + 4 g + (0..3)  (see lds_read_tr_frag for how the read works)
+__device__ __forceinline__ bf16x8_t tile_read_tr_frag(const unsigned char* smem, int byte_off, int ct, int s, int lane) {
+    const int p = lane & 15, g = lane >> 4;
+    const unsigned char* a0 = smem + byte_off + tile_at(32 * s + 4 * g + (p >> 2), 16 * ct + 4 * (p & 3));
+    const unsigned char* a1 = a0 + 16 * 128;                          // 16 rows on: the same piece order
+    s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((RWKV7_LDS s16x4_t*)(a0));
+    s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((RWKV7_LDS s16x4_t*)(a1));
+    typedef short s16x8_t __attribute__((ext_vector_type(8)));
+    s16x8_t r = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    return __builtin_bit_cast(bf16x8_t, r);
+}
+// one transposing read: lane (x, g) receives column 16 ct + x of rows row0 + 4 g + (0..3)
+__device__ __forceinline__ bf16x4_t tile_read_tr4(const unsigned char* smem, int byte_off, int row0, int ct, int lane) {
+    const int p = lane & 15, g = lane >> 4;
+    const unsigned char* a0 = smem + byte_off + tile_at(row0 + 4 * g + (p >> 2), 16 * ct + 4 * (p & 3));
+    s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((RWKV7_LDS s16x4_t*)(a0));
+    return __builtin_bit_cast(bf16x4_t, v);
+}
 
 __device__ __forceinline__ void unpack8(bf16x8_t x, float* f) {
 #pragma unroll
@@ -200,7 +232,7 @@ struct FusedArgs {
 // the exclusive cumulative decay (what RWKV7 does to a), the intra-chunk matrix Aqk keeps only j < i, and
 // its diagonal takes the bonus sum_c r_ic u_c k_ic.  a_ and b_ are not read.
 template <int MODE, bool V6 = false>
-__global__ __launch_bounds__(256, 2)
+__global__ __launch_bounds__(256, 3)
 void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restrict__ w_,
                           const bf16_t* __restrict__ k_, const bf16_t* __restrict__ v_,
                           const bf16_t* __restrict__ a_, const bf16_t* __restrict__ b_,
@@ -228,98 +260,137 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
     const int t_local = 16 * w + x;
     const int t = c * CH + t_local;
     const bool valid = t < T;
+    const bool ragged = (c + 1) * CH > T;        // uniform: only the last chunk of a sequence can be
     const int64_t row = ((cc.tok0 + t) * H + hi) * HEAD;
+    const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+    float* const tot = reinterpret_cast<float*>(smem + OFF_TOT);
 
     // ---- P0: load the chunk.  Lane (x, g) takes channels 8g..8g+7 and 32+8g..32+8g+7 of token x:
     // exactly the "plain" MFMA fragments of k-steps 0 and 1 for this wave's 16-token tile.
+    // The two 64-byte halves of a token's 128-byte row are requested back to back so that the second
+    // request finds the first one's miss in flight.  Rows past T (last chunk only) are read from the last
+    // valid row and replaced afterwards.
+    // (element offset of this lane's first piece, from a lane id: the several-bucket body calls it with an opaque
+    // copy of the lane id, so that its addresses are formed there and not kept alive from here)
+    auto first_piece = [&](int lane_) -> int64_t {
+        const int t_ = c * CH + 16 * w + (lane_ & 15);
+        return ((cc.tok0 + (t_ < T ? t_ : T - 1)) * H + hi) * HEAD + 8 * (lane_ >> 4);
+    };
+    auto load2 = [&](const bf16_t* base, int64_t at, bf16x8_t (&F)[2]) {
+        F[0] = load_frag_global(base + at, true);
+        F[1] = load_frag_global(base + at + 32, true);
+    };
+    // Decays are kept as x = -log2 of the decay (>= 0): per step from the API's w as log2(e) exp(w) =
+    // 2^(w log2 e + log2 log2 e), clamped at 87 nats (e^-87 is below FLT_MIN); then its inclusive sum over the
+    // wave's sixteen tokens.  w = -1e9 (the padding convention) gives exactly 0, a decay of exactly 1.
+    auto decays = [&](bf16x8_t (&W)[2], float (&xs)[16], float (&X)[16]) {
+        if (ragged) {                  // (the empty statement keeps this a branch: as selects it would cost every chunk)
+            asm volatile("" ::: "memory");
+            if (!valid) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) { W[0][j] = (bf16_t)(-3.0e38f); W[1][j] = (bf16_t)(-3.0e38f); }
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const float wv = (float)W[e >> 3][e & 7];
+            xs[e] = fminf(ex2(fmaf(wv, LOG2E, LOG2_LOG2E)), X_STEP_MAX);
+        }
+#pragma unroll
+        for (int e = 0; e < 16; ++e) X[e] = row_inclusive_scan(xs[e]);
+    };
+    // ... plus the totals of the waves before this one (after barrier B0)
+    auto add_prefix = [&](float (&X)[16]) {
+#pragma unroll
+        for (int ww = 0; ww < 3; ++ww) {
+            if (ww < w) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    const float4_t* src = reinterpret_cast<const float4_t*>(tot + ww * 64 + 32 * s + 8 * g);
+                    const float4_t a0 = src[0], a1 = src[1];
+                    X[8 * s + 0] += a0.x; X[8 * s + 1] += a0.y; X[8 * s + 2] += a0.z; X[8 * s + 3] += a0.w;
+                    X[8 * s + 4] += a1.x; X[8 * s + 5] += a1.y; X[8 * s + 6] += a1.z; X[8 * s + 7] += a1.w;
+                }
+            }
+        }
+    };
+
     bf16x8_t R[2], K[2], V[2], A[2], B[2];
-    float gl[16];                      // log2 decay, later its inclusive cumsum
+    float xs[16], X[16];               // -log2 decay of this lane's token per channel: the step's, the inclusive sum
     {
         bf16x8_t W[2];
-        // The two 64-byte halves of a token's 128-byte row are requested back to back so that the
-        // second request finds the first one's miss in flight.  Rows past T (last chunk only) are
-        // read from the last valid row and zeroed afterwards.
-        const int64_t row_ld = valid ? row : ((cc.tok0 + (T - 1)) * H + hi) * HEAD;
-        const int c0 = 8 * g, c1 = 32 + 8 * g;
-        W[0] = load_frag_global(w_ + row_ld + c0, true); W[1] = load_frag_global(w_ + row_ld + c1, true);
-        R[0] = load_frag_global(r_ + row_ld + c0, true); R[1] = load_frag_global(r_ + row_ld + c1, true);
-        K[0] = load_frag_global(k_ + row_ld + c0, true); K[1] = load_frag_global(k_ + row_ld + c1, true);
-        V[0] = load_frag_global(v_ + row_ld + c0, true); V[1] = load_frag_global(v_ + row_ld + c1, true);
+        const int64_t at = first_piece(lane);
+        load2(w_, at, W); load2(r_, at, R); load2(k_, at, K); load2(v_, at, V);
         if constexpr (V6) {
             A[0] = A[1] = B[0] = B[1] = load_frag_global(nullptr, false);
         } else {
-            A[0] = load_frag_global(a_ + row_ld + c0, true); A[1] = load_frag_global(a_ + row_ld + c1, true);
-            B[0] = load_frag_global(b_ + row_ld + c0, true); B[1] = load_frag_global(b_ + row_ld + c1, true);
+            load2(a_, at, A); load2(b_, at, B);
         }
-        if ((c + 1) * CH > T) {        // uniform: only the last chunk of a sequence can be ragged
+        if (ragged) {
+            asm volatile("" ::: "memory");
             if (!valid) {
                 const bf16x8_t z = load_frag_global(nullptr, false);
                 R[0] = R[1] = K[0] = K[1] = V[0] = V[1] = A[0] = A[1] = B[0] = B[1] = z;
             }
         }
-        // (rows past the end: times zero rather than a select, which the compiler turns into a branch around
-        // every one of the sixteen evaluations)
-        const float vmask = valid ? 1.f : 0.f;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-            const float wv = (float)W[e >> 3][e & 7];
-            gl[e] = vmask * fmaxf(-LOG2E * ex2(LOG2E * wv), G_MIN);           // log2 of exp(-exp(w))
-        }
+        decays(W, xs, X);
     }
-    float gstep[16];
-#pragma unroll
-    for (int e = 0; e < 16; ++e) { gstep[e] = gl[e]; gl[e] = row_inclusive_scan(gl[e]); }
-    float* tot = reinterpret_cast<float*>(smem + OFF_TOT);
-    if (x == 15) {
+    if (x == 15) {                     // the wave's last token: its totals
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
             float4_t* dst = reinterpret_cast<float4_t*>(tot + w * 64 + 32 * s + 8 * g);
-            dst[0] = float4_t{gl[8 * s + 0], gl[8 * s + 1], gl[8 * s + 2], gl[8 * s + 3]};
-            dst[1] = float4_t{gl[8 * s + 4], gl[8 * s + 5], gl[8 * s + 6], gl[8 * s + 7]};
+            dst[0] = float4_t{X[8 * s + 0], X[8 * s + 1], X[8 * s + 2], X[8 * s + 3]};
+            dst[1] = float4_t{X[8 * s + 4], X[8 * s + 5], X[8 * s + 6], X[8 * s + 7]};
         }
     }
-    __syncthreads();                                                           // B0
-    float gsum[16];                    // chunk total per channel (<= 0)
     {
-        // totals of the four waves; the prefix of waves before this one is picked by a wave-uniform
-        // branch, not by per-element selects
-        float tw[4][16];
+        // The largest of the wave's totals (the sums grow along the tokens, so it is the largest value any lane
+        // holds).  The sum of the four waves' maxima bounds every channel's chunk total from above: below one
+        // bucket, the chunk needs a single pass, and no wave has to add up the totals to know.
+        float m = X[0];
+#pragma unroll
+        for (int e = 1; e < 16; ++e) m = fmaxf(m, X[e]);
+        m = max_over_rows(m);
+        if (lane == 63) reinterpret_cast<float*>(smem + OFF_TMAX)[w] = m;
+    }
+    __syncthreads();                                                           // B0
+    add_prefix(X);
+    const float4_t tm = *reinterpret_cast<const float4_t*>(smem + OFF_TMAX);
+    const bool one_bucket = __builtin_amdgcn_readfirstlane((int)((tm.x + tm.y) + (tm.z + tm.w) < BUCKET)) != 0;
+
+    // Everything from here on exists twice: for a chunk whose decays stay inside one exponent bucket (RWKV7's own
+    // range: always) and for one that may need several passes; the choice is uniform over the workgroup.  Two
+    // bodies rather than branches inside one, so that the common one does not keep alive what only the rare
+    // one needs; the rare one loads its inputs again where it needs them a second time.
+    auto body = [&](auto single_bucket) {
+    constexpr bool SINGLE = decltype(single_bucket)::value;
+    int np = 1;                        // number of exponent buckets in this chunk (uniform over the workgroup)
+    float gsum[16];                    // several buckets: the chunk's total per channel
+    if constexpr (!SINGLE) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) gsum[e] = 0.f;
 #pragma unroll
         for (int ww = 0; ww < 4; ++ww) {
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
                 const float4_t* src = reinterpret_cast<const float4_t*>(tot + ww * 64 + 32 * s + 8 * g);
                 const float4_t a0 = src[0], a1 = src[1];
-                tw[ww][8 * s + 0] = a0.x; tw[ww][8 * s + 1] = a0.y; tw[ww][8 * s + 2] = a0.z; tw[ww][8 * s + 3] = a0.w;
-                tw[ww][8 * s + 4] = a1.x; tw[ww][8 * s + 5] = a1.y; tw[ww][8 * s + 6] = a1.z; tw[ww][8 * s + 7] = a1.w;
+                gsum[8 * s + 0] += a0.x; gsum[8 * s + 1] += a0.y; gsum[8 * s + 2] += a0.z; gsum[8 * s + 3] += a0.w;
+                gsum[8 * s + 4] += a1.x; gsum[8 * s + 5] += a1.y; gsum[8 * s + 6] += a1.z; gsum[8 * s + 7] += a1.w;
             }
         }
-        float s01[16];
+        float xmax = 0.f;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) { s01[e] = tw[0][e] + tw[1][e]; gsum[e] = s01[e] + (tw[2][e] + tw[3][e]); }
-        if (w == 1) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) gl[e] += tw[0][e];
-        } else if (w == 2) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) gl[e] += s01[e];
-        } else if (w == 3) {
-#pragma unroll
-            for (int e = 0; e < 16; ++e) gl[e] += s01[e] + tw[2][e];
-        }
+        for (int e = 0; e < 16; ++e) xmax = fmaxf(xmax, gsum[e]);
+        xmax = max_over_rows(xmax);
+        np = __builtin_amdgcn_readfirstlane((int)(xmax * (1.f / BUCKET)) + 1);
     }
-    // number of exponent buckets in this chunk (uniform over the workgroup)
-    float xmax = 0.f;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) xmax = fmaxf(xmax, -gsum[e]);
-    xmax = max_over_rows(xmax);
-    const int npass = (int)(xmax * (1.f / BUCKET)) + 1;
 
-    if (w == 0 && x == 0) {            // decay of the whole chunk per key channel
+    if (w == 3 && x == 15) {           // decay of the whole chunk per key channel: the last token's inclusive sums
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            const float4_t e0 = {ex2(gsum[8 * s + 0]), ex2(gsum[8 * s + 1]), ex2(gsum[8 * s + 2]), ex2(gsum[8 * s + 3])};
-            const float4_t e1 = {ex2(gsum[8 * s + 4]), ex2(gsum[8 * s + 5]), ex2(gsum[8 * s + 6]), ex2(gsum[8 * s + 7])};
+            const float4_t e0 = {ex2(-X[8 * s + 0]), ex2(-X[8 * s + 1]), ex2(-X[8 * s + 2]), ex2(-X[8 * s + 3])};
+            const float4_t e1 = {ex2(-X[8 * s + 4]), ex2(-X[8 * s + 5]), ex2(-X[8 * s + 6]), ex2(-X[8 * s + 7])};
             float4_t* l4 = reinterpret_cast<float4_t*>(reinterpret_cast<float*>(smem + OFF_EG) + 32 * s + 8 * g);
             l4[0] = e0; l4[1] = e1;
             if constexpr (MODE != MODE_FUSED) {
@@ -330,63 +401,48 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
     }
 
     // ---- P1: decay-scaled operands
-    float rf[16], kf[16], af[16], bf_[16];
-    unpack8(R[0], rf); unpack8(R[1], rf + 8); unpack8(K[0], kf); unpack8(K[1], kf + 8);
-    unpack8(A[0], af); unpack8(A[1], af + 8); unpack8(B[0], bf_); unpack8(B[1], bf_ + 8);
+    bf16x8_t QG[2], AG[2];
     float bonus = 0.f;                 // V6: sum_c r u k of this lane's token (rows past the end: r = k = 0)
-    if constexpr (V6) {
-        float uf[16];
-        unpack8(load_frag_global(fa.u + hi * HEAD + 8 * g, true), uf);
-        unpack8(load_frag_global(fa.u + hi * HEAD + 32 + 8 * g, true), uf + 8);
+    {
+        float rf[16], kf[16], af[16], bf_[16];
+        unpack8(R[0], rf); unpack8(R[1], rf + 8); unpack8(K[0], kf); unpack8(K[1], kf + 8);
+        unpack8(A[0], af); unpack8(A[1], af + 8); unpack8(B[0], bf_); unpack8(B[1], bf_ + 8);
+        if constexpr (V6) {
+            float uf[16];
+            unpack8(load_frag_global(fa.u + hi * HEAD + 8 * g, true), uf);
+            unpack8(load_frag_global(fa.u + hi * HEAD + 32 + 8 * g, true), uf + 8);
 #pragma unroll
-        for (int e = 0; e < 16; ++e) bonus = fmaf(rf[e] * uf[e], kf[e], bonus);
-        bonus = sum_over_rows(bonus);
-    }
-    bf16x8_t QG[2], AG[2], KG[2], BG[2];
-    auto scale_operands = [&](auto single_bucket) {
+            for (int e = 0; e < 16; ++e) bonus = fmaf(rf[e] * uf[e], kf[e], bonus);
+            bonus = sum_over_rows(bonus);
+        }
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            const float xi = -gl[e];                              // >= 0
-            // bucket 0 only; with a single bucket (the wave-uniform common case) every xi is inside it
-            const float up = (decltype(single_bucket)::value || xi < BUCKET) ? ex2(xi) : 0.f;
+            // bucket 0 only; with a single bucket every sum is inside it
+            const float up = (SINGLE || X[e] < BUCKET) ? ex2(X[e]) : 0.f;
+            const float da = ex2(xs[e] - X[e]);                   // the decay up to, not including, this token
             const int s = e >> 3, j = e & 7;
-            QG[s][j] = (bf16_t)(rf[e] * ex2(V6 ? gl[e] - gstep[e] : gl[e]));
-            AG[s][j] = (bf16_t)(af[e] * ex2(gl[e] - gstep[e]));
-            if constexpr (!decltype(single_bucket)::value) {
-                // several buckets: the end-of-chunk operands kg, bg are formed here; with one bucket they
-                // are k~, b~ times the chunk decay, which is applied to the products instead
-                const float tail = ex2(gsum[e] - gl[e]);          // <= 1
-                KG[s][j] = (bf16_t)(kf[e] * tail);
-                BG[s][j] = (bf16_t)(bf_[e] * tail);
-            }
+            QG[s][j] = (bf16_t)(rf[e] * (V6 ? da : ex2(-X[e])));
+            AG[s][j] = (bf16_t)(af[e] * da);
             K[s][j] = (bf16_t)(kf[e] * up);                       // K, B now hold k~, b~ of pass 0
             B[s][j] = (bf16_t)(bf_[e] * up);
         }
-    };
-    if (npass == 1) scale_operands(std::true_type{}); else scale_operands(std::false_type{});
+    }
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
         *reinterpret_cast<bf16x8_t*>(smem + OFF_KT + ((w * 2 + s) * 64 + lane) * 16) = K[s];
         *reinterpret_cast<bf16x8_t*>(smem + OFF_BT + ((w * 2 + s) * 64 + lane) * 16) = B[s];
-        const int col = 32 * s + 8 * g;
-        *reinterpret_cast<bf16x8_t*>(smem + OFF_QG + (t_local * LDQ + col) * 2) = QG[s];
-        *reinterpret_cast<bf16x8_t*>(smem + OFF_AG + (t_local * LDT + col) * 2) = AG[s];
-        *reinterpret_cast<bf16x8_t*>(smem + OFF_V + (t_local * LDT + col) * 2) = V[s];
+        const int at = tile_at(t_local, 32 * s + 8 * g);
+        *reinterpret_cast<bf16x8_t*>(smem + OFF_AG + at) = AG[s];
+        *reinterpret_cast<bf16x8_t*>(smem + OFF_V + at) = V[s];
     }
     __syncthreads();                                                           // B1
-    bf16x8_t DOr[2];                   // MODE_BWD: this lane's row of dO, on its way to the tile V leaves at B3
-    if constexpr (BWD) {
-        if (fa.d_o != nullptr && valid) {
-            DOr[0] = load_frag_global(fa.d_o + row + 8 * g, true);
-            DOr[1] = load_frag_global(fa.d_o + row + 32 + 8 * g, true);
-        } else {
-            DOr[0] = DOr[1] = load_frag_global(nullptr, false);
-        }
-    }
 
     // ---- P2: the four intra-chunk matrices, block row w.  D[j][i] = sum_c kb[j][c] qa[i][c], so a
     // lane holds four consecutive j of one i: an 8-byte piece of a sigma fragment of the [i][j] matrix.
-    const float4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+    // (V leaves its tile for the registers first: the tile's place is taken by Aak behind the next barrier.)
+    bf16x8_t Vtr[2];
+    Vtr[0] = tile_read_tr_frag(smem, OFF_V, w, 0, lane);
+    Vtr[1] = tile_read_tr_frag(smem, OFF_V, w, 1, lane);
     float4_t acc_qk[4], acc_qb[4], acc_ak[4], acc_ab[4];
     float4_t diagX = zero4;                 // D layout of X = Aab[w][w] (rows i, column j)
 #pragma unroll
@@ -394,27 +450,49 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         if (J <= w) { acc_qk[J] = zero4; acc_qb[J] = zero4; acc_ak[J] = zero4; acc_ab[J] = zero4; }
     }
     bf16x8_t Qp[2] = {QG[0], QG[1]}, Ap[2] = {AG[0], AG[1]};
-    for (int p = 0; p < npass; ++p) {
-        if (p > 0) {                        // rare: tokens whose cumulative decay lies in bucket p
-            __syncthreads();
-            const float base = BUCKET * (float)p;
+    for (int p = 0; p < np; ++p) {
+        if constexpr (!SINGLE) {
+            if (p > 0) {                    // rare: tokens whose cumulative decay lies in bucket p
+                __syncthreads();
+                const float base = BUCKET * (float)p;
+                float xs2[16], X2[16];
+                bf16x8_t W2[2], R2[2], K2[2], A2[2], B2[2];
+                int lane_o = lane;
+                asm volatile("" : "+v"(lane_o));
+                const int64_t at = first_piece(lane_o);
+                load2(w_, at, W2); load2(r_, at, R2); load2(k_, at, K2);
+                if constexpr (V6) {
+                    A2[0] = A2[1] = B2[0] = B2[1] = load_frag_global(nullptr, false);
+                } else {
+                    load2(a_, at, A2); load2(b_, at, B2);
+                }
+                if (ragged) {
+                    asm volatile("" ::: "memory");
+                    if (!valid) R2[0] = R2[1] = K2[0] = K2[1] = A2[0] = A2[1] = B2[0] = B2[1] = load_frag_global(nullptr, false);
+                }
+                decays(W2, xs2, X2);
+                add_prefix(X2);
+                float rf[16], kf[16], af[16], bf_[16];
+                unpack8(R2[0], rf); unpack8(R2[1], rf + 8); unpack8(K2[0], kf); unpack8(K2[1], kf + 8);
+                unpack8(A2[0], af); unpack8(A2[1], af + 8); unpack8(B2[0], bf_); unpack8(B2[1], bf_ + 8);
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const float xi = -gl[e], xe = xi + gstep[e];      // xe = -(exclusive cumsum)
-                const float up = (xi >= base && xi < base + BUCKET) ? ex2(xi - base) : 0.f;
-                const int s = e >> 3, j = e & 7;
-                K[s][j] = (bf16_t)(kf[e] * up);
-                B[s][j] = (bf16_t)(bf_[e] * up);
-                Qp[s][j] = V6 ? (bf16_t)(xe >= base ? rf[e] * ex2(base - xe) : 0.f)
-                              : (bf16_t)(xi >= base ? rf[e] * ex2(base - xi) : 0.f);
-                Ap[s][j] = (bf16_t)(xe >= base ? af[e] * ex2(base - xe) : 0.f);
-            }
+                for (int e = 0; e < 16; ++e) {
+                    const float xi = X2[e], xe = xi - xs2[e];        // xe: up to, not including, this token
+                    const float up = (xi >= base && xi < base + BUCKET) ? ex2(xi - base) : 0.f;
+                    const int s = e >> 3, j = e & 7;
+                    K[s][j] = (bf16_t)(kf[e] * up);
+                    B[s][j] = (bf16_t)(bf_[e] * up);
+                    Qp[s][j] = V6 ? (bf16_t)(xe >= base ? rf[e] * ex2(base - xe) : 0.f)
+                                  : (bf16_t)(xi >= base ? rf[e] * ex2(base - xi) : 0.f);
+                    Ap[s][j] = (bf16_t)(xe >= base ? af[e] * ex2(base - xe) : 0.f);
+                }
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                *reinterpret_cast<bf16x8_t*>(smem + OFF_KT + ((w * 2 + s) * 64 + lane) * 16) = K[s];
-                *reinterpret_cast<bf16x8_t*>(smem + OFF_BT + ((w * 2 + s) * 64 + lane) * 16) = B[s];
+                for (int s = 0; s < 2; ++s) {
+                    *reinterpret_cast<bf16x8_t*>(smem + OFF_KT + ((w * 2 + s) * 64 + lane) * 16) = K[s];
+                    *reinterpret_cast<bf16x8_t*>(smem + OFF_BT + ((w * 2 + s) * 64 + lane) * 16) = B[s];
+                }
+                __syncthreads();
             }
-            __syncthreads();
         }
 #pragma unroll
         for (int J = 0; J < 4; ++J) {
@@ -438,51 +516,47 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
             if constexpr (!V6) diagX = mfma_bf16(Ap[s], lds_read_frag(smem, OFF_BT, w * 2 + s, lane), diagX);
     }
     float4_t diagXT = zero4;                // D layout of X^T (rows j, column i)
-    {
-        // causal masks on the diagonal block: j <= i for Aqk/Aqb, j < i for Aak/Aab (j = 4g+e, i = x)
+    // causal masks on the diagonal block: j <= i for Aqk/Aqb, j < i for Aak/Aab (j = 4g+e, i = x)
 #pragma unroll
-        for (int J = 0; J < 4; ++J) {
-            if (J == w) {
+    for (int J = 0; J < 4; ++J) {
+        if (J == w) {
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int jj = 4 * g + e;
-                    if (jj > x) { acc_qk[J][e] = 0.f; acc_qb[J][e] = 0.f; }
-                    if constexpr (V6) { if (jj == x) acc_qk[J][e] = bonus; }
-                    if (jj >= x) { acc_ak[J][e] = 0.f; acc_ab[J][e] = 0.f; }
-                    if (x >= jj) diagX[e] = 0.f;          // here rows are i = 4g+e, column j = x: keep j < i
-                }
-                diagXT = acc_ab[J];
+            for (int e = 0; e < 4; ++e) {
+                const int jj = 4 * g + e;
+                if (jj > x) { acc_qk[J][e] = 0.f; acc_qb[J][e] = 0.f; }
+                if constexpr (V6) { if (jj == x) acc_qk[J][e] = bonus; }
+                if (jj >= x) { acc_ak[J][e] = 0.f; acc_ab[J][e] = 0.f; }
+                if (x >= jj) diagX[e] = 0.f;          // here rows are i = 4g+e, column j = x: keep j < i
+            }
+            diagXT = acc_ab[J];
+        }
+    }
+    __syncthreads();                                                           // Bx: every wave has taken its V
+#pragma unroll
+    for (int J = 0; J < 4; ++J) {
+        if (J <= w) {
+            const int f = fidx(w, J >> 1);
+            const int off = ((f * 64 + lane) * 8 + 4 * (J & 1)) * 2;
+            *reinterpret_cast<bf16x4_t*>(smem + OFF_AQK + off) = pack4(acc_qk[J]);
+            *reinterpret_cast<bf16x4_t*>(smem + OFF_AQB + off) = pack4(acc_qb[J]);
+            *reinterpret_cast<bf16x4_t*>(smem + OFF_AAK + off) = pack4(acc_ak[J]);
+            if (J < w) {
+                // block (w, J), row-major [i][j]: lane holds i = x, j = 4g..4g+3
+                *reinterpret_cast<bf16x4_t*>(smem + OFF_AAB + lidx(w, J) * 512 + (x * 16 + 4 * g) * 2) = pack4(acc_ab[J]);
             }
         }
-#pragma unroll
-        for (int J = 0; J < 4; ++J) {
-            if (J <= w) {
-                const int f = fidx(w, J >> 1);
-                const int off = ((f * 64 + lane) * 8 + 4 * (J & 1)) * 2;
-                *reinterpret_cast<bf16x4_t*>(smem + OFF_AQK + off) = pack4(acc_qk[J]);
-                *reinterpret_cast<bf16x4_t*>(smem + OFF_AQB + off) = pack4(acc_qb[J]);
-                *reinterpret_cast<bf16x4_t*>(smem + OFF_AAK + off) = pack4(acc_ak[J]);
-                if (J < w) {
-                    // block (w, J), row-major [i][j]: lane holds i = x, j = 4g..4g+3
-                    *reinterpret_cast<bf16x4_t*>(smem + OFF_AAB + bidx(w, J) * 512 + (x * 16 + 4 * g) * 2) = pack4(acc_ab[J]);
-                }
-            }
-        }
-        if ((w & 1) == 0) {                 // the j-tile right of the diagonal shares a fragment: zero it
-            const int off = ((fidx(w, w >> 1) * 64 + lane) * 8 + 4) * 2;
-            const bf16x4_t z = pack4(zero4);
-            *reinterpret_cast<bf16x4_t*>(smem + OFF_AQK + off) = z;
-            *reinterpret_cast<bf16x4_t*>(smem + OFF_AQB + off) = z;
-            *reinterpret_cast<bf16x4_t*>(smem + OFF_AAK + off) = z;
-        }
+    }
+    if ((w & 1) == 0) {                     // the j-tile right of the diagonal shares a fragment: zero it
+        const int off = ((fidx(w, w >> 1) * 64 + lane) * 8 + 4) * 2;
+        const bf16x4_t z = pack4(zero4);
+        *reinterpret_cast<bf16x4_t*>(smem + OFF_AQK + off) = z;
+        *reinterpret_cast<bf16x4_t*>(smem + OFF_AQB + off) = z;
+        *reinterpret_cast<bf16x4_t*>(smem + OFF_AAK + off) = z;
     }
     __syncthreads();                                                           // B2
 
     // ---- P3: T1 = Aak V for this wave's 16 value columns (kept in registers), and the inverse of
     // the diagonal block: (I - N)^-1 = (I + N)(I + N^2)(I + N^4)(I + N^8), N strictly lower 16x16.
-    bf16x8_t Vtr[2];
-    Vtr[0] = lds_read_tr_frag(smem, OFF_V, LDT, w, 0, lane);
-    Vtr[1] = lds_read_tr_frag(smem, OFF_V, LDT, w, 1, lane);
     float4_t t1[4];
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
@@ -511,10 +585,18 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
     // DmT lane (column i' = x, rows j' = 4g..): DmT[j'][i'] = Dinv[i'][j'] -> row i' of Dinv, columns 4g..4g+3
     if constexpr (!V6) *reinterpret_cast<bf16x4_t*>(smem + OFF_DI + w * 512 + (x * 16 + 4 * g) * 2) = pack4(DmT);
     __syncthreads();                                                           // B3 (all T1 reads of Aak done)
-    if constexpr (BWD) {               // V is in registers (Vtr) everywhere: its tile takes dO
+    // qg, in the registers since P1, takes the place of Aak: it is read behind B4
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
-            *reinterpret_cast<bf16x8_t*>(smem + OFF_V + (t_local * LDT + 32 * s + 8 * g) * 2) = DOr[s];
+    for (int s = 0; s < 2; ++s)
+        *reinterpret_cast<bf16x8_t*>(smem + OFF_QG + tile_at(t_local, 32 * s + 8 * g)) = QG[s];
+    bf16x8_t DOr[2];                   // MODE_BWD: this lane's row of dO, on its way to the tile ag leaves at B4
+    if constexpr (BWD) {
+        if (fa.d_o != nullptr && valid) {
+            DOr[0] = load_frag_global(fa.d_o + row + 8 * g, true);
+            DOr[1] = load_frag_global(fa.d_o + row + 32 + 8 * g, true);
+        } else {
+            DOr[0] = DOr[1] = load_frag_global(nullptr, false);
+        }
     }
 
     // ---- P4: W = M ag and U = M T1 without forming M = (I - Aab)^-1: block forward substitution
@@ -526,7 +608,7 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         bf16x4_t Xw[4], Xu[4];
 #pragma unroll
         for (int I = 0; I < 4; ++I) {
-            float4_t aw = unpack4(lds_read_tr4(smem, OFF_AG, LDT, 16 * I, w, lane));   // ag[16I+4g+e][16w+x]
+            float4_t aw = unpack4(tile_read_tr4(smem, OFF_AG, 16 * I, w, lane));   // ag[16I+4g+e][16w+x]
             // The 16x16x16 chain starts from zero and T1 (a 16x16x32 result) is added by the VALU: a
             // 16x16x16 MFMA that takes the result of a 16x16x32 MFMA as its accumulator input less than five
             // wait states after it reads two of the four registers before they are written (measured on
@@ -537,7 +619,7 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
             for (int J = 0; J < 3; ++J) {
                 if (J < I) {
                     const bf16x4_t a4 = *reinterpret_cast<const bf16x4_t*>(
-                        smem + OFF_AAB + bidx(I, J) * 512 + (x * 16 + 4 * g) * 2);
+                        smem + OFF_AAB + lidx(I, J) * 512 + (x * 16 + 4 * g) * 2);
                     aw = mfma_bf16_k16(a4, Xw[J], aw);
                     au = mfma_bf16_k16(a4, Xu[J], au);
                 }
@@ -549,16 +631,41 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
             Xu[I] = pack4(uacc[I]);
         }
     }
-    const bool single = npass == 1;
-    if constexpr (BWD) { if (single) __syncthreads(); }        // the dO tile is complete (several buckets: B4)
-    if (!single) {
-        __syncthreads();                                                       // B4
-        // kg, bg row-major into the space the inverse no longer needs
+    __syncthreads();                                                           // B4: qg is in place, ag is done with
+    if constexpr (BWD) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+            *reinterpret_cast<bf16x8_t*>(smem + OFF_DO + tile_at(t_local, 32 * s + 8 * g)) = DOr[s];
+    }
+    if constexpr (!SINGLE) {
+        // several buckets: the end-of-chunk operands kg = k e^{G - g_i}, bg likewise, as tiles where k~, b~ lay
+        float xs2[16], X2[16];
+        bf16x8_t W2[2], K2[2], B2[2];
+        int lane_o = lane;
+        asm volatile("" : "+v"(lane_o));
+        const int64_t at = first_piece(lane_o);
+        load2(w_, at, W2); load2(k_, at, K2);
+        if constexpr (V6) B2[0] = B2[1] = load_frag_global(nullptr, false); else load2(b_, at, B2);
+        if (ragged) {
+            asm volatile("" ::: "memory");
+            if (!valid) K2[0] = K2[1] = B2[0] = B2[1] = load_frag_global(nullptr, false);
+        }
+        decays(W2, xs2, X2);
+        add_prefix(X2);
+        float kf[16], bf_[16];
+        unpack8(K2[0], kf); unpack8(K2[1], kf + 8); unpack8(B2[0], bf_); unpack8(B2[1], bf_ + 8);
+        bf16x8_t KG[2], BG[2];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const float tail = ex2(X2[e] - gsum[e]);              // <= 1
+            KG[e >> 3][e & 7] = (bf16_t)(kf[e] * tail);
+            BG[e >> 3][e & 7] = (bf16_t)(bf_[e] * tail);
+        }
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            const int col = 32 * s + 8 * g;
-            *reinterpret_cast<bf16x8_t*>(smem + OFF_KG + (t_local * LDT + col) * 2) = KG[s];
-            *reinterpret_cast<bf16x8_t*>(smem + OFF_BG + (t_local * LDT + col) * 2) = BG[s];
+            const int at = tile_at(t_local, 32 * s + 8 * g);
+            *reinterpret_cast<bf16x8_t*>(smem + OFF_KG + at) = KG[s];
+            *reinterpret_cast<bf16x8_t*>(smem + OFF_BG + at) = BG[s];
         }
         __syncthreads();                                                       // B5
     }
@@ -590,7 +697,7 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
 #pragma unroll
         for (int s = 0; s <= it / 2; ++s)
             if constexpr (!V6) acc = mfma_bf16(Ws[s], lds_read_frag(smem, OFF_AQB, fidx(it, s), lane), acc);
-        const bf16x4_t q4 = *reinterpret_cast<const bf16x4_t*>(smem + OFF_QG + ((16 * it + x) * LDQ + 16 * w + 4 * g) * 2);
+        const bf16x4_t q4 = *reinterpret_cast<const bf16x4_t*>(smem + OFF_QG + tile_at(16 * it + x, 16 * w + 4 * g));
         acc.x += (float)q4[0]; acc.y += (float)q4[1]; acc.z += (float)q4[2]; acc.w += (float)q4[3];
         if constexpr (MODE == MODE_FUSED) qth[it] = pack4(acc);
         else *reinterpret_cast<bf16x4_t*>(qt + nn * 4096 + ((it * 4 + w) * 64 + lane) * 4) = pack4(acc);
@@ -605,10 +712,11 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
 #pragma unroll
         for (int s = 0; s <= it / 2; ++s)
             acc = mfma_bf16(lds_read_frag(smem, OFF_AQB, fidx(it, s), lane), Ws[s], acc);
-        const bf16x4_t q4 = lds_read_tr4(smem, OFF_QG, LDQ, 16 * it, w, lane);   // qg[16it+4g+e][16w+x]
+        const bf16x4_t q4 = tile_read_tr4(smem, OFF_QG, 16 * it, w, lane);   // qg[16it+4g+e][16w+x]
         acc.x += (float)q4[0]; acc.y += (float)q4[1]; acc.z += (float)q4[2]; acc.w += (float)q4[3];
         qn[it] = acc;
     }
+    if constexpr (SINGLE) __syncthreads();                     // the dO tile is complete (several buckets: B5)
     // (Qt^T dO)[c][v] = sum_i Qt[i][c] dO[i][v] for key tile w, all four value tiles
     const bf16x8_t qts[2] = {pack_sigma(qn[0], qn[1]), pack_sigma(qn[2], qn[3])};
 #pragma unroll
@@ -616,7 +724,7 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         float4_t acc = zero4;
 #pragma unroll
         for (int s = 0; s < 2; ++s)
-            acc = mfma_bf16(qts[s], lds_read_tr_frag(smem, OFF_V, LDT, vt, s, lane), acc);
+            acc = mfma_bf16(qts[s], tile_read_tr_frag(smem, OFF_DO, vt, s, lane), acc);
         *reinterpret_cast<bf16x4_t*>(qt + nn * 4096 + ((vt * 4 + w) * 64 + lane) * 4) = pack4(acc);
     }
     }
@@ -625,45 +733,40 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
     // from the fragment arrays of P2 and the chunk decay eG[c] multiplies the results (in fused mode
     // not even that: it is applied once to the new state).
     const float* egl = reinterpret_cast<const float*>(smem + OFF_EG);
-    auto end_of_chunk_products = [&](auto single_bucket) {
-        constexpr bool SINGLE = decltype(single_bucket)::value;
 #pragma unroll
-        for (int ct = 0; ct < 4; ++ct) {
-            float4_t accp = zero4, accq = zero4;
+    for (int ct = 0; ct < 4; ++ct) {
+        float4_t accp = zero4, accq = zero4;
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                const bf16x8_t bgt = SINGLE ? lds_read_tr_frag_tokens(smem, OFF_BT, ct, s, lane)
-                                            : lds_read_tr_frag(smem, OFF_BG, LDT, ct, s, lane);
-                const bf16x8_t kgt = SINGLE ? lds_read_tr_frag_tokens(smem, OFF_KT, ct, s, lane)
-                                            : lds_read_tr_frag(smem, OFF_KG, LDT, ct, s, lane);
-                accq = mfma_bf16(kgt, Vtr[s], accq);
-                if constexpr (!V6) {
-                    accp = mfma_bf16(Ws[s], bgt, accp);
-                    accq = mfma_bf16(bgt, Us[s], accq);
-                }
-            }
-            if constexpr (MODE == MODE_FUSED) {
-                pph[ct] = pack4(accp); qcacc[ct] = accq;
-            } else {
-                if constexpr (SINGLE) {
-                    const float ex = egl[16 * ct + x];                                   // column c of accp
-                    const float4_t e4 = *reinterpret_cast<const float4_t*>(egl + 16 * ct + 4 * g);   // rows c
-                    accp = accp * ex;
-                    accq = accq * e4;
-                }
-                *reinterpret_cast<bf16x4_t*>(pp + nn * 4096 + ((ct * 4 + w) * 64 + lane) * 4) = pack4(accp);
-                *reinterpret_cast<bf16x4_t*>(qc + nn * 4096 + ((w * 4 + ct) * 64 + lane) * 4) = pack4(accq);
+        for (int s = 0; s < 2; ++s) {
+            const bf16x8_t bgt = SINGLE ? lds_read_tr_frag_tokens(smem, OFF_BT, ct, s, lane)
+                                        : tile_read_tr_frag(smem, OFF_BG, ct, s, lane);
+            const bf16x8_t kgt = SINGLE ? lds_read_tr_frag_tokens(smem, OFF_KT, ct, s, lane)
+                                        : tile_read_tr_frag(smem, OFF_KG, ct, s, lane);
+            accq = mfma_bf16(kgt, Vtr[s], accq);
+            if constexpr (!V6) {
+                accp = mfma_bf16(Ws[s], bgt, accp);
+                accq = mfma_bf16(bgt, Us[s], accq);
             }
         }
-    };
-    if (single) end_of_chunk_products(std::true_type{}); else end_of_chunk_products(std::false_type{});
+        if constexpr (MODE == MODE_FUSED) {
+            pph[ct] = pack4(accp); qcacc[ct] = accq;
+        } else {
+            if constexpr (SINGLE) {
+                const float ex = egl[16 * ct + x];                                   // column c of accp
+                const float4_t e4 = *reinterpret_cast<const float4_t*>(egl + 16 * ct + 4 * g);   // rows c
+                accp = accp * ex;
+                accq = accq * e4;
+            }
+            *reinterpret_cast<bf16x4_t*>(pp + nn * 4096 + ((ct * 4 + w) * 64 + lane) * 4) = pack4(accp);
+            *reinterpret_cast<bf16x4_t*>(qc + nn * 4096 + ((w * 4 + ct) * 64 + lane) * 4) = pack4(accq);
+        }
+    }
 
     if constexpr (MODE == MODE_FUSED) {
         // ---- apply the chunk to the state.  State at the start of the chunk: chunk 0 takes h0, later
         // chunks wait for the previous chunk's workgroup (lower block index, hence already dispatched)
-        // to publish value tile w.  Data and counter are device-scope accesses; the producer's
-        // s_waitcnt between the two makes the counter the last thing to become visible.  The loads are
-        // issued before the exchange below and collected after it.
+        // to publish value tile w as a marked image (handoff_marks).  The loads of a first look at the slot
+        // are issued inside the exchange below and collected after it.
         float4_t h[4];
         const int slot_in = (c - 1) & 1, slot_out = c & 1;
         float* const hin = fa.hbuf + ((int64_t)slot_in * BH + bh) * 4096 + (w * 4 * 64 + lane) * 4;
@@ -696,8 +799,8 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         // other halves), so the halves go through LDS into the tiles that the chains no longer read.
         __syncthreads();
         if (c != 0) state_load_issue(hin, cin, h, car);      // a first look at the slot, collected behind the exchange below
-        bf16_t* fq = reinterpret_cast<bf16_t*>(smem + OFF_AG);       // [4 tiles][2 k-steps][2 halves][64][4]
-        bf16_t* fp = reinterpret_cast<bf16_t*>(smem + OFF_V);
+        bf16_t* fq = reinterpret_cast<bf16_t*>(smem + OFF_FQ);       // [4 tiles][2 k-steps][2 halves][64][4]
+        bf16_t* fp = reinterpret_cast<bf16_t*>(smem + OFF_FP);
 #pragma unroll
         for (int m = 0; m < 4; ++m) {
             *reinterpret_cast<bf16x4_t*>(fq + ((m * 4 + w) * 64 + lane) * 4) = qth[m];
@@ -748,8 +851,7 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         split_sigma(h[2], h[3], bhi[1], blo[1]);
         const float* egs = reinterpret_cast<const float*>(smem + OFF_EG);
         float4_t hn[4];
-        auto new_state = [&](auto single_bucket) {      // a wave-uniform branch, not per-element selects
-            constexpr bool SINGLE = decltype(single_bucket)::value;
+        {
 #pragma unroll
             for (int ct = 0; ct < 4; ++ct) {
                 const float4_t e4 = *reinterpret_cast<const float4_t*>(egs + 16 * ct + 4 * g);
@@ -766,8 +868,7 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
                 }
                 hn[ct] = SINGLE ? e4 * acc : acc;
             }
-        };
-        if (single) new_state(std::true_type{}); else new_state(std::false_type{});
+        }
         // send the new state on its way first (the next chunk needs it); the counter that announces it
         // is bumped after the output products below, which run while the stores are in flight
         if (c + 1 < NT) {
@@ -796,19 +897,21 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
                 acc = mfma_bf16(a8, bhi[s], acc);
                 acc = mfma_bf16(a8, blo[s], acc);
             }
-            *reinterpret_cast<bf16x4_t*>(smem + OFF_QG + ((16 * w + x) * LDQ + 16 * it + 4 * g) * 2) = pack4(acc);
+            *reinterpret_cast<bf16x4_t*>(smem + OFF_OT + tile_at(16 * w + x, 16 * it + 4 * g)) = pack4(acc);
         }
         __syncthreads();
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
             // token 16 w + x, values 32 s + 8 g .. + 7
-            const bf16x4_t lo = lds_read_tr4(smem, OFF_QG, LDQ, 32 * s + 4 * g, w, lane);
-            const bf16x4_t hi4 = lds_read_tr4(smem, OFF_QG, LDQ, 32 * s + 4 * g + 4, w, lane);
+            const bf16x4_t lo = tile_read_tr4(smem, OFF_OT, 32 * s + 4 * g, w, lane);
+            const bf16x4_t hi4 = tile_read_tr4(smem, OFF_OT, 32 * s + 4 * g + 4, w, lane);
             if (valid)
                 *reinterpret_cast<bf16x8_t*>(fa.o + row + 32 * s + 8 * g) =
                     bf16x8_t{lo[0], lo[1], lo[2], lo[3], hi4[0], hi4[1], hi4[2], hi4[3]};
         }
     }
+    };   // body
+    if (one_bucket) body(std::true_type{}); else body(std::false_type{});
 }
 
 // The scan of the two-kernel form: one workgroup per (batch, head), wave = 16 value columns.  State
