@@ -152,14 +152,17 @@ __device__ __forceinline__ void state_load_wait(float4_t (&h)[4], uint32_t& car)
 // word a 3-bit field (bits 8+3j .. 10+3j for the j-th such float, j = 0..7) is replaced by a mark; the bits
 // that stood there travel in the same field of the carrier, whose low 8 bits are its own mark, and the reader
 // puts them back: the state crosses the hand-off bit for bit.  The marks of chunk c are the fields of
-//     E(c) = S(1 + (c / 2) mod 7) ^ tag32,   S(v) = v in every 3-bit field and v | v << 3 in the low byte,
-// so the fields of two images that follow each other in a slot differ (as do those seven uses apart), and a
-// cleared slot holds S(0) ^ tag32 = tag32 in every 4-byte piece, which is no chunk's mark in any field.  An
-// image half arrived still shows an old field somewhere: two fields per 16-byte word catch a word torn at
-// 8 bytes or coarser (the memory system moves 32 bytes or more at a time).
+//     E(c) = S(c / 2) ^ tag32,   S(u) = 1 + u mod 7 in every 3-bit field and 1 + u mod 255 in the low byte,
+// so the fields of two images that follow each other in a slot differ, and a cleared slot holds
+// S = 0, i.e. tag32, in every 4-byte piece, which is no chunk's mark in any field.  An image half arrived
+// still shows its predecessor's field somewhere: two fields per 16-byte word catch a word torn at 8 bytes or
+// coarser (the memory system moves 32 bytes or more at a time).  A reader ahead of its turn may find an image
+// in the slot that is several uses old (with few heads the chip holds the workgroups of many chunk positions
+// at once); the 3-bit fields repeat every seven uses, the carrier's byte only every 255, which is further
+// than any reader can be ahead.
 __device__ __forceinline__ uint32_t handoff_marks(unsigned long long tag, int c) {
-    const uint32_t v = 1u + (uint32_t)(c >> 1) % 7u;
-    return (v * 0x24924900u | v * 9u) ^ (uint32_t)tag;
+    const uint32_t u = (uint32_t)(c >> 1);
+    return ((1u + u % 7u) * 0x24924900u | (1u + u % 255u)) ^ (uint32_t)tag;
 }
 __device__ __forceinline__ uint32_t bfi(uint32_t mask, uint32_t a, uint32_t b) { return (a & mask) | (b & ~mask); }
 // marks into the image, the bits they replace into the carrier (returned)
