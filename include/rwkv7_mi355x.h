@@ -41,7 +41,9 @@
 extern "C" {
 #endif
 
-#define RWKV7_ABI_VERSION 1
+/* 2: the one-kernel forward's workspace holds a status record, two state slots per (batch, head) and their
+ * carriers (sizes from the *_workspace_bytes functions as before); rwkv7_set_giveup_notice; RWKV6 float32 gradients */
+#define RWKV7_ABI_VERSION 2
 
 /* element type of r, w, k, v, a, b, o and the input gradients */
 #define RWKV7_DTYPE_BF16 0
@@ -78,7 +80,7 @@ const char* rwkv7_status_string(int status);
  * (:46-120).  Writes o [B,T,H,64] (`dtype`) and, if ht != NULL, the final state.
  * bf16 runs the fused chunked MFMA kernel (one workgroup per 64-token chunk; the
  * state travels from chunk to chunk through the workspace) and needs a workspace of
- * rwkv7_fwd_workspace_bytes() (a few MB: two state slots and four counters per
+ * rwkv7_fwd_workspace_bytes() (a few MB: two state slots of 17 KiB per
  * (batch, head)); f32 runs the chunked float32 kernel (16-token chunks on the float32
  * matrix cores, one workgroup per (batch, head) with the state in registers; float32
  * arithmetic throughout, the accuracy of the reference's native loop) and needs none (ws
@@ -107,8 +109,8 @@ int rwkv7_fwd(const void* r, const void* w, const void* k, const void* v,
  * around the call -- code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc -- and so cannot provide rwkv7_fwd's workspace: the same forward,
  * same arguments and results, with the workspace taken from a static device array
- * inside the library (8.01 MiB, held on every GPU the library is loaded on until the
- * process ends).  That array holds the one-kernel form's hand-off slots and counters
+ * inside the library (8.5 MiB, held on every GPU the library is loaded on until the
+ * process ends).  That array holds the one-kernel form's hand-off slots and status record
  * for up to RWKV7_NOALLOC_MAX_BH (batch, head) sequences, so B*H beyond that is refused
  * with RWKV7_ERR_TOO_LARGE; T is not limited.  bf16 with T > 12 always takes the
  * one-kernel chunked form here (rwkv7_fwd prefers two kernels below 96 sequences, whose
@@ -119,7 +121,7 @@ int rwkv7_fwd(const void* r, const void* w, const void* k, const void* v,
  * calls on one GPU share the array: two of them that overlap in time (different
  * streams, or graphs replayed concurrently) race and give wrong results; calls on one
  * stream are ordered and safe.  Nothing in the array needs clearing between calls:
- * every launch tags its counters with a fresh 64-bit value (see rwkv7_fwd_status). */
+ * every launch marks the states it hands over with a fresh tag (see rwkv7_fwd_status). */
 #define RWKV7_NOALLOC_MAX_BH 256
 int rwkv7_fwd_noalloc(const void* r, const void* w, const void* k, const void* v,
                       const void* a, const void* b,
@@ -142,8 +144,9 @@ int rwkv7_fwd_noalloc(const void* r, const void* w, const void* k, const void* v
  * rwkv7_fwd_status_offset), rwkv7_fwd_varlen (rwkv7_fwd_varlen_status_offset), and the
  * two-kernel form, whose summary launch writes a record that can only read "done".
  * The offset functions return RWKV7_NO_STATUS_RECORD for shapes and dtypes whose call
- * runs no chunked kernel (T <= 12, float32, float16; K = V = 128).  No counterpart in the reference,
- * whose kernels do not communicate. */
+ * runs no chunked kernel (T <= 12, float32, float16).  They take no head size: a call at K = V = 128
+ * writes no record either (its kernels use no workspace), so do not ask for one there.  No counterpart in
+ * the reference, whose kernels do not communicate. */
 #define RWKV7_NO_STATUS_RECORD ((size_t)-1)
 #define RWKV7_FWD_DONE      0   /* the launch that wrote the record did not give up */
 #define RWKV7_FWD_GAVE_UP   1   /* a hand-off wait timed out: o and ht hold NaN */
@@ -152,6 +155,12 @@ size_t rwkv7_fwd_status_offset(int B, int T, int H, int dtype);
 size_t rwkv7_fwd_varlen_status_offset(int n_seq, int T_total, int H, int dtype);
 /* `record`: HOST pointer to a copy of the 16-byte record.  Returns RWKV7_FWD_* or RWKV7_ERR_NULL_POINTER. */
 int rwkv7_fwd_status(const void* record);
+/* The same news without a copy or a synchronisation: a word of pinned host memory that the device can write
+ * (hipHostMalloc), set to 0 by the caller.  A one-kernel forward that gives up stores a non-zero value there
+ * (besides its status record), which the host sees on a plain read some time after; a caller looks at the word
+ * before its next call, say.  One word per process, NULL to take it away; the caller keeps the memory alive for
+ * as long as it is registered.  No counterpart in the reference. */
+int rwkv7_set_giveup_notice(unsigned long long* host_word);
 
 /* ---- initial states gathered through a map -----------------------------------------
  * The reference's RWKV6 operator lets several batch rows start from one of a few

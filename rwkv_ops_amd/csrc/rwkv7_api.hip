@@ -125,6 +125,11 @@ size_t rwkv7_fwd_status_offset(int B, int T, int H, int dtype) {
                                    : rwkv7::fwd_chunk_status_offset(B, T, H);
 }
 
+int rwkv7_set_giveup_notice(unsigned long long* host_word) {
+    rwkv7::giveup_notice().store(host_word, std::memory_order_release);
+    return RWKV7_OK;
+}
+
 int rwkv7_fwd_status(const void* record) {
     if (!record) return RWKV7_ERR_NULL_POINTER;
     const unsigned long long* rec = static_cast<const unsigned long long*>(record);

@@ -226,6 +226,7 @@ struct FusedArgs {
     float* hbuf;               // [2][B*H][4 value tiles][4 key tiles][64 lanes][4] float hand-off slots
     uint32_t* hcar;            // [2][B*H][4 value tiles][64 lanes] the slots' carriers (see handoff_marks)
     unsigned long long tag;    // this launch's random 64-bit tag: the slots need no clearing (see launch_fwd_fused)
+    unsigned long long* notice; // nullable: a word in host memory that a wave which gives up writes the tag into (see rwkv7_set_giveup_notice)
     unsigned long long* status; // nullable: [0] = give-up flag (== tag: a hand-off wait timed out), [1] = tag of the launch
 };
 
@@ -833,6 +834,8 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
                         if (now - t0 > WAIT_LIMIT_TICKS ||
                             __hip_atomic_load(fa.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == fa.tag) {
                             __hip_atomic_store(fa.status, fa.tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            if (fa.notice != nullptr)
+                                __hip_atomic_store(fa.notice, fa.tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                             ok = false;
                             break;
                         }
@@ -1438,6 +1441,11 @@ size_t fwd_fused_workspace_bytes(int B, int T, int H, bool varlen) {
     return fwd_fused_bytes((size_t)B * H) + (varlen ? chunk_items_bytes(B, T) : 0);
 }
 
+std::atomic<unsigned long long*>& giveup_notice() {
+    static std::atomic<unsigned long long*> word{nullptr};
+    return word;
+}
+
 hipError_t launch_fwd_fused(const SeqArgs& p, void* ws, hipStream_t stream) {
     const int BH = p.B * p.H;
     const int64_t nchunks = chunk_records(p.B, p.T, p.H, p.cu != nullptr);
@@ -1460,6 +1468,7 @@ hipError_t launch_fwd_fused(const SeqArgs& p, void* ws, hipStream_t stream) {
     // readers of a head's last images clear them (see there).
     fa.tag = next_launch_tag();
     fa.u = static_cast<const bf16_t*>(p.u6);
+    fa.notice = giveup_notice().load(std::memory_order_acquire);
     return p.u6 ? launch_summary_kernel<MODE_FUSED, true>(p, nchunks, nullptr, nullptr, nullptr, nullptr, nullptr, L, fa, stream)
                 : launch_summary_kernel<MODE_FUSED, false>(p, nchunks, nullptr, nullptr, nullptr, nullptr, nullptr, L, fa, stream);
 }

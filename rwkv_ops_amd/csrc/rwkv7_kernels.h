@@ -1,6 +1,8 @@
 // Internal launch interface between the C ABI (rwkv7_api.hip) and the kernel files.
 #pragma once
 
+#include <atomic>
+
 #include <hip/hip_runtime.h>
 #include <stddef.h>
 #include <stdint.h>
@@ -46,6 +48,8 @@ constexpr size_t fwd_fused_bytes(size_t bh) { return 256 + 2 * bh * (4096 * 4 + 
 size_t fwd_fused_status_offset(int B, int T, int H, bool varlen = false);
 size_t fwd_chunk_status_offset(int B, int T, int H, bool varlen = false);
 hipError_t launch_fwd_fused(const SeqArgs& p, void* ws, hipStream_t stream);
+// the word (device-accessible host memory, or null) that a fused forward which gives up writes its tag into
+std::atomic<unsigned long long*>& giveup_notice();
 // its two halves: the parallel per-chunk summaries (reads r..b, fills ws) and the serial scan
 // (reads ws and h0, writes o and ht)
 hipError_t launch_fwd_chunk_summary(const SeqArgs& p, void* ws, hipStream_t stream);

@@ -31,7 +31,7 @@ from typing import Optional
 import torch
 
 from ..rwkv7 import _lib
-from ..rwkv7.op import _dtype_code, _on_device, _ptr, _require_gpu, _stream_ptr
+from ..rwkv7.op import _as_state_map, _dtype_code, _on_device, _ptr, _require_gpu, _stream_ptr
 
 __all__ = ["RWKVKernelOperator", "get_rwkv6_kernel"]
 
@@ -150,13 +150,9 @@ class RWKVKernelOperator:
                 if n_state not in (1, B):
                     raise ValueError("state_map cannot be inferred: give it explicitly")
             else:
-                if isinstance(state_map, (list, tuple)):
-                    state_map = torch.tensor(state_map, dtype=torch.int32)
-                if state_map.dtype not in (torch.int32, torch.int64) or tuple(state_map.shape) != (B,):
-                    raise ValueError(f"state_map must be an int tensor or list of shape [{B}]")
-                if bool((state_map < 0).any()) or bool((state_map >= n_state).any()):
-                    raise ValueError(f"state_map entries must lie in [0, {n_state})")
-                smap = state_map.to(device=r.device, dtype=torch.int32).contiguous()
+                # a list or a CPU tensor is checked (torch_rwkv_kernel.py:293-297); a tensor on the device is taken
+                # as it is, without a read-back that would stall the stream (the kernels clamp what they read)
+                smap = _as_state_map(state_map, B, n_state, r.device)
         elif state_map is not None:
             raise ValueError("state_map needs an init_state to index")
 

@@ -1,1 +1,1 @@
-from .op import generalized_delta_rule, rwkv7_decode_step, HEAD_SIZE  # noqa: F401
+from .op import generalized_delta_rule, rwkv7_decode_step, last_forward_status, HEAD_SIZE  # noqa: F401

@@ -36,7 +36,7 @@ HEAD_SIZE = 64
 # K = V = 128 has the decode step, a chunked bf16 forward of its own and the float32 recurrent forward and backward
 HEAD_SIZES = (64, 128)
 
-__all__ = ["generalized_delta_rule", "rwkv7_decode_step", "HEAD_SIZE"]
+__all__ = ["generalized_delta_rule", "rwkv7_decode_step", "last_forward_status", "HEAD_SIZE"]
 
 
 def _dtype_code(dt: torch.dtype) -> int:
@@ -107,8 +107,23 @@ def _direct(*tensors) -> bool:
     return True
 
 
+def last_forward_status(synchronize: bool = False) -> str:
+    """"ok" or "gave_up": whether a one-kernel chunked forward launched from this process has stopped waiting for
+    a state hand-off and poisoned its outputs with NaN since the last look (the look clears the mark).  Reads one
+    word of pinned host memory; with ``synchronize`` the devices are synchronised first, so that every forward
+    launched so far has had its say.  The forward calls look themselves, at their start, and raise
+    ``ForwardGaveUp`` -- this function is for a caller that wants to know before its next call."""
+    if synchronize and torch.cuda.is_available():
+        torch.cuda.synchronize()
+    word = _lib.giveup_notice()
+    gave_up = int(word[0]) != 0
+    word[0] = 0
+    return "gave_up" if gave_up else "ok"
+
+
 def _fwd_impl(r, w, k, v, a, b, h0, want_state, state_map=None):
     lib = _lib.load()
+    _lib.raise_if_gave_up()
     B, T, H, N = r.shape
     o = torch.empty_like(r)
     ht = torch.empty((B, H, N, N) if want_state else (0,), dtype=torch.float32, device=r.device)
@@ -215,8 +230,11 @@ def _fwd_setup_context(ctx, inputs, output):
 
 def _fwd_backward(ctx, d_o, d_ht):
     r, w, k, v, a, b, h0_arg, state_map = ctx.saved_tensors
-    # with a map the backward kernels see the gathered states; dh0 is scattered back below
-    h0 = h0_arg if state_map is None else h0_arg.index_select(0, state_map.long())
+    # with a map the backward kernels see the gathered states; dh0 is scattered back below.  The map is clamped
+    # as the kernels clamp it: a map that came on the device was never checked (no read-back), and an entry out
+    # of range must not trip a device-side assertion here either
+    rows = None if state_map is None else state_map.long().clamp_(0, h0_arg.shape[0] - 1)
+    h0 = h0_arg if rows is None else h0_arg.index_select(0, rows)
     dt = r.dtype
     d_ht_c = None
     if ctx.want_state and d_ht is not None and d_ht.numel() > 0:
@@ -241,7 +259,7 @@ def _fwd_backward(ctx, d_o, d_ht):
     g0 = None
     if h0 is not None and ctx.needs_input_grad[6]:
         if state_map is not None:
-            g0 = torch.zeros_like(h0_arg).index_add_(0, state_map.long(), dh0)
+            g0 = torch.zeros_like(h0_arg).index_add_(0, rows, dh0)
         else:
             g0 = dh0.sum(0, keepdim=True) if h0.shape[0] != dh0.shape[0] else dh0
     return dr.to(dt), dw.to(dt), dk.to(dt), dv.to(dt), da.to(dt), db.to(dt), g0, None, None
@@ -253,6 +271,7 @@ rwkv7_fwd.register_autograd(_fwd_backward, setup_context=_fwd_setup_context)
 # ---- packed sequences (cu_seqlens)
 def _fwd_varlen_impl(r, w, k, v, a, b, h0, want_state, cu):
     lib = _lib.load()
+    _lib.raise_if_gave_up()
     _, T, H, N = r.shape
     n_seq = cu.numel() - 1
     o = torch.empty_like(r)
@@ -573,7 +592,9 @@ def generalized_delta_rule(
     ``out`` has the dtype of the inputs for bfloat16, float16 and float32 inputs, whatever T is (the
     reference's kernel path returns bfloat16 for all of them, torch_op.py:451-455,486); float16 sequences of
     more than 12 tokens are computed from bfloat16-rounded operands, as the reference does, and ``out`` is
-    rounded back to float16.
+    rounded back to float16 (an output beyond float16's range, 65504, becomes inf there).  The final state is
+    float32 for every input dtype (the reference casts it to the input dtype, torch_op.py:487-488): a decode loop
+    can feed it back without loss.
 
     ``w`` is the raw decay argument: the per-step decay is ``exp(-exp(w))``
     (torch_op.py:433-434), so padded positions use ``w += (1 - mask) * -1e9`` together

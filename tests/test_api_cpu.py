@@ -103,3 +103,19 @@ def test_custom_ops_have_shape_functions():
         assert ops.rwkv7_decode(*step, h0).shape == step[0].shape
         pool = torch.empty(7, H, 64, 64, device="cuda")
         assert ops.rwkv7_decode_pool(*step, pool, torch.empty(B, dtype=torch.int32, device="cuda")).shape == step[0].shape
+
+
+def test_forward_calls_look_at_the_giveup_word():
+    """Both forward implementations call ``_lib.raise_if_gave_up`` before they launch (the GPU test sets the word)."""
+    import inspect
+    from rwkv_ops_amd.rwkv7 import op
+    for fn in (op._fwd_impl, op._fwd_varlen_impl):
+        assert "raise_if_gave_up" in inspect.getsource(fn)
+
+
+def test_backward_clamps_a_state_map():
+    """The autograd backward gathers and scatters through a clamped copy of the map (a device map is never checked)."""
+    import inspect
+    from rwkv_ops_amd.rwkv7 import op
+    src = inspect.getsource(op._fwd_backward)
+    assert "clamp_(0, h0_arg.shape[0] - 1)" in src and "index_add_(0, rows" in src

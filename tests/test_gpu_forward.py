@@ -81,3 +81,15 @@ def test_recurrent_kernel_matches_oracle(device, dtype, B, T, H):
     o2, _ = torch.ops.rwkv_ops_amd.rwkv7_fwd_recurrent(r, w, k, v, a, b, None, False)
     o2_ref = orc.generalized_delta_rule(*[x.float() for x in xs[:6]], None, output_final_state=False)
     assert rel_l2(o2, o2_ref) < TOL[dtype]
+
+
+@pytest.mark.parametrize("T", [1, 8, 40])                      # decode kernel, recurrent kernel, chunked kernels
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_return_dtypes(device, dtype, T):
+    """``out`` comes back in the dtype of the inputs and the final state in float32, whatever the kernel: a choice
+    that differs from the reference's kernel path, which returns a bfloat16 ``out`` for every input dtype and casts
+    the state to the input dtype (torch_op.py:451-455,486-488), and is pinned here."""
+    xs = [x.to(device) for x in make_inputs(2, T, 3, 64, seed=90 + T, dtype=dtype)]
+    o, s = rwkv_ops_amd.generalized_delta_rule(*xs)
+    assert o.dtype == dtype and s.dtype == torch.float32
+    assert o.shape == xs[0].shape and s.shape == (2, 3, 64, 64)

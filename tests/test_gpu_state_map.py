@@ -92,3 +92,23 @@ def test_decode_pool_in_place(device):
     assert torch.equal(got[untouched], pool[untouched])          # other slots: bitwise unchanged
     with pytest.raises(ValueError):
         rwkv_ops_amd.rwkv7_decode_step(*[x[:, 0].to(device) for x in xs[:6]], dpool, state_map=[1, 1, 2, 3])
+
+
+def test_a_bad_device_map_does_not_fault(device):
+    """A map that arrives on the device is never read back, so nothing checks it: the kernels clamp what they read,
+    and the backward's gather and scatter on the host side clamp the same way (no device-side index assertion)."""
+    B, T, H, n_state = 3, 70, 2, 4
+    xs = make_inputs(B, T, H, 64, seed=411, dtype=torch.bfloat16)
+    pool = _pool(n_state, H, seed=5)
+    bad = torch.tensor([-3, 2, 99], dtype=torch.int32, device=device)
+    good = bad.clamp(0, n_state - 1)
+    outs = []
+    for m in (bad, good):
+        dev = [x.to(device).requires_grad_(True) for x in xs[:6]]
+        p = pool.to(device).requires_grad_(True)
+        o, s = rwkv_ops_amd.generalized_delta_rule(*dev, initial_state=p, state_map=m)
+        (o.float().sum() + s.sum()).backward()
+        torch.cuda.synchronize()
+        outs.append([o, s, p.grad] + [d.grad for d in dev])
+    for x, y in zip(*outs):
+        assert torch.equal(x, y)

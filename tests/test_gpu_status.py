@@ -58,3 +58,38 @@ def test_status_after_a_packed_forward(device):
     assert rc == 0
     torch.cuda.synchronize()
     assert _status(lib, ws, off)[0] == _lib.FWD_DONE
+
+
+def test_giveup_notice_reaches_python(device):
+    """The pinned host word that a forward which gives up writes into: the next forward call raises, the call
+    after it runs (the word is cleared by the look), and ``last_forward_status`` reports and clears it too.
+    No wait is made to time out on the GPU: the host plays the device's part and sets the word."""
+    import rwkv_ops_amd
+    xs = [x.to(device) for x in make_inputs(2, 200, 48, 64, seed=73, dtype=torch.bfloat16)]
+    o, s = rwkv_ops_amd.generalized_delta_rule(*xs)                       # registers the word on first use
+    assert rwkv_ops_amd.last_forward_status(synchronize=True) == "ok"
+    word = _lib.giveup_notice()
+    assert word.is_pinned() and int(word[0]) == 0
+    word[0] = 12345
+    with pytest.raises(_lib.ForwardGaveUp):
+        rwkv_ops_amd.generalized_delta_rule(*xs)
+    o2, s2 = rwkv_ops_amd.generalized_delta_rule(*xs)
+    assert torch.equal(o2, o) and torch.equal(s2, s)
+    word[0] = 7
+    assert rwkv_ops_amd.last_forward_status() == "gave_up"
+    assert rwkv_ops_amd.last_forward_status() == "ok"
+
+
+def test_the_device_can_write_the_notice_word(device):
+    """The word is host memory that kernels can store to: a device-side fill of a view of it is seen by the host."""
+    word = _lib.giveup_notice()
+    word[0] = 0
+    import ctypes as c
+    hip = c.CDLL("libamdhip64.so")
+    dev_ptr = c.c_void_p()
+    assert hip.hipHostGetDevicePointer(c.byref(dev_ptr), c.c_void_p(word.data_ptr()), 0) == 0
+    assert dev_ptr.value == word.data_ptr()          # the same address on both sides: what the library is given
+    assert hip.hipMemsetD32(dev_ptr, 0x01010101, 2) == 0
+    torch.cuda.synchronize()
+    assert int(word[0]) == 0x0101010101010101
+    word[0] = 0
