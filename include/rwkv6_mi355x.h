@@ -48,12 +48,13 @@ int rwkv6_fwd_recurrent(const void* r, const void* k, const void* v, const void*
 /* ---- backward of the call without a state ---------------------------------------------------------
  * Replaces RWKV_6.backward (/root/reference/rwkv_ops/rwkv6_kernel/torch_rwkv_kernel.py:93-152: the four
  * backward kernels of wkv6_cuda.cu and the sum of gu over the batch): given r, k, v, w, u and d_y
- * ([B, T, H, 64], bf16), writes dr, dk, dv, dw (same shape and type; dw is the gradient with respect to the
+ * ([B, T, H, 64], bf16 or float32), writes dr, dk, dv, dw (same shape and type; dw is the gradient with respect to the
  * w argument, the decay being exp(-exp(w))) and du (float32 [H, 64], already summed over the batch).  The
  * initial state is zero and no final state is returned, as in the reference's differentiable path.  The
  * state-path gradients come from the RWKV7 backward kernels run on the operands read one token ahead
- * (r_{t+1} against k_t, v_t, w_t); the bonus term's gradient is added by an epilogue kernel.  bf16 only
- * (f32: RWKV7_ERR_UNSUPPORTED). */
+ * (r_{t+1} against k_t, v_t, w_t); the bonus term's gradient is added by an epilogue kernel.  float32 tensors
+ * run the float32 kernels and get float32-accurate gradients, as the reference's float32 kernel gives them
+ * (torch_rwkv_kernel.py:137); float16: RWKV7_ERR_UNSUPPORTED. */
 size_t rwkv6_bwd_workspace_bytes(int B, int T, int H, int dtype);
 int rwkv6_bwd(const void* r, const void* k, const void* v, const void* w, const void* u,
               const void* d_y,

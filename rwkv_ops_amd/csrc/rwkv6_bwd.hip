@@ -36,12 +36,13 @@ void rwkv6_bwd_prologue_kernel(int* __restrict__ cu, u32x4_t* __restrict__ zeros
 // the primed terms being zero where the state path has none (t = 0 for dr, t = T-1 for the others; the
 // buffers hold the dummy sequences' values or nothing there).  dk, dv, dw are corrected in place.
 // du[h][c] = sum over batch and tokens of r k s: summed per workgroup, then one atomic per channel.
+template <typename E>
 __global__ __launch_bounds__(256)
-void rwkv6_bwd_epilogue_kernel(const bf16_t* __restrict__ r, const bf16_t* __restrict__ k,
-                               const bf16_t* __restrict__ v, const bf16_t* __restrict__ u,
-                               const bf16_t* __restrict__ dy, const bf16_t* __restrict__ dr_state,
-                               bf16_t* __restrict__ dr, bf16_t* __restrict__ dk, bf16_t* __restrict__ dv,
-                               bf16_t* __restrict__ dw, float* __restrict__ du, int T, int H, int state_path)
+void rwkv6_bwd_epilogue_kernel(const E* __restrict__ r, const E* __restrict__ k,
+                               const E* __restrict__ v, const E* __restrict__ u,
+                               const E* __restrict__ dy, const E* __restrict__ dr_state,
+                               E* __restrict__ dr, E* __restrict__ dk, E* __restrict__ dv,
+                               E* __restrict__ dw, float* __restrict__ du, int T, int H, int state_path)
 {
     __shared__ float part[4][HEAD];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
@@ -61,10 +62,10 @@ void rwkv6_bwd_epilogue_kernel(const bf16_t* __restrict__ r, const bf16_t* __res
         const float dr0 = (state_path && !first) ? (float)dr_state[row - (int64_t)H * HEAD] : 0.f;
         const float dk0 = (state_path && !last) ? (float)dk[row] : 0.f;
         const float dv0 = (state_path && !last) ? (float)dv[row] : 0.f;
-        dr[row] = (bf16_t)(dr0 + uc * kc * s);
-        dk[row] = (bf16_t)(dk0 + uc * rc * s);
-        dv[row] = (bf16_t)(dv0 + q * gc);
-        if (!state_path || last) dw[row] = (bf16_t)0.f;
+        dr[row] = (E)(dr0 + uc * kc * s);
+        dk[row] = (E)(dk0 + uc * rc * s);
+        dv[row] = (E)(dv0 + q * gc);
+        if (!state_path || last) dw[row] = (E)0.f;
         du_acc = fmaf(rc * kc, s, du_acc);
     }
     part[wv][lane] = du_acc;
@@ -82,18 +83,24 @@ size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 }  // namespace
 
 // workspace: [cu table][zeros][dr of the state path][da, db dump][RWKV7 backward workspace]
-size_t rwkv6_bwd_workspace_bytes(int B, int T, int H) {
-    const size_t tensor = align256((size_t)B * T * H * HEAD * 2);
+size_t rwkv6_bwd_workspace_bytes(int B, int T, int H, int dtype) {
+    const bool f32 = dtype == RWKV7_DTYPE_F32;
+    const size_t tensor = align256((size_t)B * T * H * HEAD * (f32 ? 4 : 2));
     size_t n = align256((size_t)2 * B * 4) + 3 * tensor;
-    if (T > 1) n += bwd_chunk_workspace_bytes(2 * B - 1, B * T - 1, H, true);
+    if (T > 1) n += f32 ? bwd_chunk_f32_workspace_bytes(2 * B - 1, B * T - 1, H, true)
+                        : bwd_chunk_workspace_bytes(2 * B - 1, B * T - 1, H, true);
     return n;
 }
 
 hipError_t launch_rwkv6_bwd(const void* r, const void* k, const void* v, const void* w, const void* u,
                             const void* dy, void* dr, void* dk, void* dv, void* dw, float* du,
-                            int B, int T, int H, void* ws, hipStream_t stream)
+                            int B, int T, int H, int dtype, void* ws, hipStream_t stream)
 {
-    const size_t tensor = align256((size_t)B * T * H * HEAD * 2);
+    // float32 tensors: the same plan on the chunked float32 backward (every product on the float32 matrix cores),
+    // so that float32 callers get float32 gradients as the reference's float32 kernel gives them
+    // (/root/reference/rwkv_ops/rwkv6_kernel/torch_rwkv_kernel.py:137)
+    const bool f32 = dtype == RWKV7_DTYPE_F32;
+    const size_t tensor = align256((size_t)B * T * H * HEAD * (f32 ? 4 : 2));
     unsigned char* base = static_cast<unsigned char*>(ws);
     int* cu = reinterpret_cast<int*>(base);
     unsigned char* zeros = base + align256((size_t)2 * B * 4);
@@ -110,20 +117,25 @@ hipError_t launch_rwkv6_bwd(const void* r, const void* k, const void* v, const v
             cu, reinterpret_cast<u32x4_t*>(zeros), n16, B, T);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
-        const int64_t ahead = (int64_t)H * HEAD * 2;          // one token, in bytes
+        const int64_t ahead = (int64_t)H * HEAD * (f32 ? 4 : 2);          // one token, in bytes
         BwdArgs p;
         p.r = static_cast<const unsigned char*>(r) + ahead; p.w = w; p.k = k; p.v = v; p.a = zeros; p.b = zeros;
         p.h0 = nullptr; p.h0_batch_stride = 0;
         p.dO = static_cast<const unsigned char*>(dy) + ahead; p.dht = nullptr;
         p.dr = dr_state; p.dw = dw; p.dk = dk; p.dv = dv; p.da = dump; p.db = dump; p.dh0 = nullptr;
-        p.B = 2 * B - 1; p.T = B * T - 1; p.H = H; p.dtype = RWKV7_DTYPE_BF16; p.cu = cu;
-        e = launch_bwd_chunk(p, bws, stream);
+        p.B = 2 * B - 1; p.T = B * T - 1; p.H = H; p.dtype = dtype; p.cu = cu;
+        e = f32 ? launch_bwd_chunk_f32(p, bws, stream) : launch_bwd_chunk(p, bws, stream);
         if (e != hipSuccess) return e;
     }
     const int nblk = (T + 63) / 64;
-    rwkv6_bwd_epilogue_kernel<<<dim3((unsigned)(B * H * nblk)), dim3(256), 0, stream>>>(
-        (const bf16_t*)r, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)u, (const bf16_t*)dy,
-        (const bf16_t*)dr_state, (bf16_t*)dr, (bf16_t*)dk, (bf16_t*)dv, (bf16_t*)dw, du, T, H, T > 1 ? 1 : 0);
+    if (f32)
+        rwkv6_bwd_epilogue_kernel<float><<<dim3((unsigned)(B * H * nblk)), dim3(256), 0, stream>>>(
+            (const float*)r, (const float*)k, (const float*)v, (const float*)u, (const float*)dy,
+            (const float*)dr_state, (float*)dr, (float*)dk, (float*)dv, (float*)dw, du, T, H, T > 1 ? 1 : 0);
+    else
+        rwkv6_bwd_epilogue_kernel<bf16_t><<<dim3((unsigned)(B * H * nblk)), dim3(256), 0, stream>>>(
+            (const bf16_t*)r, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)u, (const bf16_t*)dy,
+            (const bf16_t*)dr_state, (bf16_t*)dr, (bf16_t*)dk, (bf16_t*)dv, (bf16_t*)dw, du, T, H, T > 1 ? 1 : 0);
     return hipGetLastError();
 }
 

@@ -529,15 +529,15 @@ int rwkv6_fwd_recurrent(const void* r, const void* k, const void* v, const void*
 }
 
 size_t rwkv6_bwd_workspace_bytes(int B, int T, int H, int dtype) {
-    if (dtype != RWKV7_DTYPE_BF16 || B < 1 || T < 1 || H < 1) return 0;
-    return rwkv7::rwkv6_bwd_workspace_bytes(B, T, H);
+    if ((dtype != RWKV7_DTYPE_BF16 && dtype != RWKV7_DTYPE_F32) || B < 1 || T < 1 || H < 1) return 0;
+    return rwkv7::rwkv6_bwd_workspace_bytes(B, T, H, dtype);
 }
 
 int rwkv6_bwd(const void* r, const void* k, const void* v, const void* w, const void* u, const void* d_y,
               void* dr, void* dk, void* dv, void* dw, float* du,
               int B, int T, int H, int K, int V, int dtype, void* ws, size_t ws_bytes, void* stream)
 {
-    if (dtype == RWKV7_DTYPE_F32) return RWKV7_ERR_UNSUPPORTED;
+    if (dtype == RWKV7_DTYPE_F16) return RWKV7_ERR_UNSUPPORTED;
     int rc = check_seq(r, w, k, v, r, r, nullptr, 0, dr, nullptr, B, T, H, K, V, dtype);
     if (rc != RWKV7_OK) return rc;
     // the state path runs as 2B - 1 packed sequences over B*T - 1 tokens
@@ -545,9 +545,9 @@ int rwkv6_bwd(const void* r, const void* k, const void* v, const void* w, const 
     if (!u || !d_y || !dk || !dv || !dw || !du) return RWKV7_ERR_NULL_POINTER;
     if (!aligned16(u) || !aligned16(d_y) || !aligned16(dk) || !aligned16(dv) || !aligned16(dw) || !aligned16(du))
         return RWKV7_ERR_ALIGNMENT;
-    const size_t need = rwkv7::rwkv6_bwd_workspace_bytes(B, T, H);
+    const size_t need = rwkv7::rwkv6_bwd_workspace_bytes(B, T, H, dtype);
     if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return RWKV7_ERR_WORKSPACE;
-    return (int)rwkv7::launch_rwkv6_bwd(r, k, v, w, u, d_y, dr, dk, dv, dw, du, B, T, H, ws,
+    return (int)rwkv7::launch_rwkv6_bwd(r, k, v, w, u, d_y, dr, dk, dv, dw, du, B, T, H, dtype, ws,
                                         static_cast<hipStream_t>(stream));
 }
 

@@ -78,19 +78,17 @@ class _Rwkv6Function(torch.autograd.Function):
         r, k, v, w, u = ctx.saved_tensors
         B, T, C = r.shape
         H = ctx.H
-        dt = r.dtype
-        bf = torch.bfloat16
-        # the backward kernels are bf16: float32 operands are rounded for the backward only
-        xs = [x if x.dtype == bf else x.to(bf) for x in (r, k, v, w, u)]
-        g = gy.to(bf).contiguous()
+        dt = r.dtype                       # bfloat16 or float32: the kernels of that type (float32 gradients for
+        code = _dtype_code(dt)             # float32 tensors, torch_rwkv_kernel.py:137)
+        g = gy.to(dt).contiguous()
         lib = _lib.load()
-        grads = [torch.empty((B, T, C), dtype=bf, device=r.device) for _ in range(4)]
+        grads = [torch.empty((B, T, C), dtype=dt, device=r.device) for _ in range(4)]
         du = torch.empty((H, HEAD_SIZE), dtype=torch.float32, device=r.device)
         with _on_device(r.device):
-            ws_bytes = lib.rwkv6_bwd_workspace_bytes(B, T, H, _lib.DTYPE_BF16)
+            ws_bytes = lib.rwkv6_bwd_workspace_bytes(B, T, H, code)
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=r.device)
-            rc = lib.rwkv6_bwd(*[_ptr(x) for x in xs], _ptr(g), *[_ptr(x) for x in grads], _ptr(du),
-                               B, T, H, HEAD_SIZE, HEAD_SIZE, _lib.DTYPE_BF16, _ptr(ws), ws_bytes,
+            rc = lib.rwkv6_bwd(*[_ptr(x) for x in (r, k, v, w, u)], _ptr(g), *[_ptr(x) for x in grads], _ptr(du),
+                               B, T, H, HEAD_SIZE, HEAD_SIZE, code, _ptr(ws), ws_bytes,
                                _stream_ptr(r.device))
         _lib.check(rc, "rwkv6_bwd")
         dr, dk, dv, dw = (x.to(dt) for x in grads)

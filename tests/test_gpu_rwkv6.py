@@ -131,22 +131,23 @@ def test_dtype_conventions(device):
 
 
 # The bf16 chunked formulation costs the RWKV7 gradients 3e-3 .. 6e-3 relative L2 (tests/test_gpu_backward.py);
-# the RWKV6 backward runs the same kernels and gets the same thresholds.
-@pytest.mark.parametrize("B,T,H", [(1, 1, 2), (2, 70, 2), (1, 300, 3), (2, 130, 40)])
+# the bf16 RWKV6 backward runs the same kernels and gets the same thresholds.  float32 tensors get float32
+# gradients from the float32 kernels (as the reference's float32 kernel gives them, torch_rwkv_kernel.py:137):
+# 1e-4 on unrounded float32 inputs; du is summed with float atomics, whose order varies (1e-4 still).
+@pytest.mark.parametrize("B,T,H", [(1, 1, 2), (2, 70, 2), (1, 300, 3), (2, 130, 40), (3, 17, 2), (2, 12, 3)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_gradients_match_oracle_autograd(device, B, T, H, dtype):
     xs = make_inputs(B, T, H, seed=8700 + T, dtype=dtype)
     g = torch.Generator().manual_seed(T)
     dy = torch.randn(B, T, H * N, generator=g).to(dtype)
-    if dtype == torch.float32:        # the backward kernels are bf16: compare on values that bf16 holds exactly
-        xs = [x.to(torch.bfloat16).float() for x in xs[:5]] + xs[5:]
-        dy = dy.to(torch.bfloat16).float()
     leaves = [x.to(device).requires_grad_(True) for x in xs[:5]]
     y, none = rwkv_ops_amd.RWKV6_OP(64, 4096)(*leaves)
     assert none is None and y.dtype == dtype
     got = torch.autograd.grad((y.float() * dy.to(device).float()).sum(), leaves, allow_unused=True)
     ref = o6.gradients(*xs[:5], dy)
     tol = {"dr": 6e-3, "dk": 6e-3, "dv": 6e-3, "dw": 8e-3, "du": 6e-3}
+    if dtype == torch.float32:
+        tol = {name: 1e-4 for name in tol}
     errs = {}
     for name, a_, b_ in zip(tol, got, ref):
         assert a_.dtype == dtype and a_.shape == b_.shape
