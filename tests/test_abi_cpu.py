@@ -133,11 +133,13 @@ def test_rwkv6_argument_errors_do_not_launch():
 
     def bwd(u=x, dy=x, du=x, dtype=0, ws=None, ws_bytes=0):
         return lib.rwkv6_bwd(x, x, x, x, u, dy, x, x, x, x, du, 2, 100, 2, 64, 64, dtype, ws, ws_bytes, None)
-    assert bwd(dtype=1) == -8                            # float32 backward is not built
+    assert bwd(dtype=2) == -8                            # float16 backward is not built
+    assert bwd(dtype=1) == -6                            # float32: built, and it wants its workspace
     assert bwd(u=None) == -1 and bwd(dy=None) == -1 and bwd(du=None) == -1
     assert bwd() == -6
     assert lib.rwkv6_bwd_workspace_bytes(2, 8, 2, 0) > 3 * 2 * 8 * 2 * 64 * 2
-    assert lib.rwkv6_bwd_workspace_bytes(2, 8, 2, 1) == 0
+    assert lib.rwkv6_bwd_workspace_bytes(2, 8, 2, 1) > 3 * 2 * 8 * 2 * 64 * 4
+    assert lib.rwkv6_bwd_workspace_bytes(2, 8, 2, 2) == 0
 
 
 def test_float16_is_a_dtype_only_where_a_kernel_reads_it():
