@@ -50,6 +50,34 @@ EXEC_FLOPS_SOURCE = ("profiles/fwd_chunk_prefill_mfma_counters.txt (SQ_INSTS_VAL
                      "token-head; a constant, not measured in this run)")
 
 
+# The two constants above describe the kernels as they were when the profiles were taken: the digest of the
+# kernel sources (sources_digest() below) at that time.  The JSON line carries this digest next to the digest of
+# the sources in the tree and of the loaded library, so a reader sees whether the constants still belong to
+# the code that was timed.
+CONSTANTS_SOURCES_DIGEST = "unset"
+
+
+def sources_digest():
+    """sha256 (first 16 hex digits) over the kernel sources and the C-ABI headers, in name order."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    files = sorted(glob.glob(os.path.join(ROOT, "rwkv_ops_amd", "csrc", "*.hip")) +
+                   glob.glob(os.path.join(ROOT, "rwkv_ops_amd", "csrc", "*.h")) +
+                   glob.glob(os.path.join(ROOT, "include", "*.h")))
+    for f in files:
+        h.update(os.path.basename(f).encode())
+        with open(f, "rb") as fh:
+            h.update(fh.read())
+    return h.hexdigest()[:16]
+
+
+def file_digest(path):
+    import hashlib
+    with open(path, "rb") as fh:
+        return hashlib.sha256(fh.read()).hexdigest()[:16]
+
+
 def algorithmic_bytes_prefill(B, T, H):
     # r, w, k, v, a, b read + o written (bf16), state read + written (float32)
     return 7 * B * T * H * N * 2 + 2 * B * H * N * N * 4
@@ -529,6 +557,10 @@ def main():
                   "ms": ms_rwkv6, "tokens_per_s": B * T / (ms_rwkv6 * 1e-3), "algorithmic_bytes": rwkv6_bytes,
                   "frac_of_hbm_peak": rwkv6_bytes / (ms_rwkv6 * 1e-3) / HBM_PEAK},
         "cpu_baseline": cpu,
+        "build": {"library": os.path.relpath(_lib.LIB_PATH, ROOT), "library_sha256_16": file_digest(_lib.LIB_PATH),
+                  "abi_version": int(lib.rwkv7_abi_version()), "sources_sha256_16": sources_digest(),
+                  "profile_constants_taken_at_sources_sha256_16": CONSTANTS_SOURCES_DIGEST,
+                  "profile_constants_current": sources_digest() == CONSTANTS_SOURCES_DIGEST},
         "wall_ms_per_step": wall_ms,
         "device": props.name,
     }
