@@ -526,7 +526,7 @@ def main():
                    "backward_ms": ms_packed_bwd, "backward_tokens_per_s": B * T / (ms_packed_bwd * 1e-3)},
         "long_sequence": {"workload": f"BASELINE config 3: one sequence, B={Bl} T={Tl} H={Hl} bf16, zero initial state, the "
                                       f"last {padl} tokens masked by w += (1-mask)*-1e9 (rwkv7_fwd: per-chunk summaries, "
-                                      "then the value-split scan, the form for fewer than 96 heads)",
+                                      "then the value-split scan, the form for fewer than 72 sequences)",
                           "ms": ms_long, "tokens_per_s": Bl * Tl / (ms_long * 1e-3),
                           "algorithmic_bytes": long_bytes,
                           "frac_of_hbm_peak": long_bytes / (ms_long * 1e-3) / HBM_PEAK,

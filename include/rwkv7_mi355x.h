@@ -113,7 +113,7 @@ int rwkv7_fwd(const void* r, const void* w, const void* k, const void* v,
  * process ends).  That array holds the one-kernel form's hand-off slots and status record
  * for up to RWKV7_NOALLOC_MAX_BH (batch, head) sequences, so B*H beyond that is refused
  * with RWKV7_ERR_TOO_LARGE; T is not limited.  bf16 with T > 12 always takes the
- * one-kernel chunked form here (rwkv7_fwd prefers two kernels below 96 sequences, whose
+ * one-kernel chunked form here (rwkv7_fwd prefers two kernels below 72 sequences, whose
  * workspace grows with T); T == 1, T <= 12, float32, float16 and K = V = 128 take the
  * same kernels as in rwkv7_fwd, which need no workspace.  The call itself allocates
  * nothing and calls no allocating routine; its first call on a device looks the

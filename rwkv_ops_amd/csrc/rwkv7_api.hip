@@ -98,9 +98,10 @@ namespace {
 // The one-kernel forward keeps a few chunks of every (batch, head) in flight, which pays when there are
 // enough sequences to fill the chip; with few, long sequences the chain of state hand-offs is the
 // critical path and the two-kernel form (parallel summaries, then a scan) is faster.
-// (measured at T = 4096: 64 sequences 114 us against 140 us fused, 96 sequences 216 us against 179 us,
-// 128 sequences 260 us against 183 us; at T = 16384: 64 sequences 472 us against 665 us)
-bool use_fused_forward(int B, int H) { return (int64_t)B * H >= 96; }
+// (measured at T = 4096: 64 sequences 114 us against 140 us fused, 72 sequences 168 us against 150 us,
+// 96 sequences 216 us against 179 us; at T = 16384: 64 sequences 472 us against 665 us, 80 sequences 777 us
+// against 684 us)
+bool use_fused_forward(int B, int H) { return (int64_t)B * H >= 72; }
 // A handful of tokens per sequence (speculative-decoding verification, very short prompts) is faster one
 // token at a time with the state in registers than through the 64-token chunk machinery, whatever the
 // number of sequences: B*H = 2560, T = 2 / 8 / 16 / 32: 17 / 30 / 49 / 89 us against 46 / 46 / 47 / 49 us

@@ -163,7 +163,7 @@ def test_packed_sequences_by_reset_tokens(device):
 
 
 # The two-kernel form through its own entry points (rwkv7_fwd_chunk_summary + rwkv7_fwd_chunk_scan), which
-# rwkv7_fwd only takes for B*H < 96: up to 128 sequences the scan is the value-split kernel (four workgroups
+# rwkv7_fwd only takes for B*H < 72: up to 128 sequences the scan is the value-split kernel (four workgroups
 # per head), above that the one-workgroup-per-head kernel.  Both against the oracle, any B*H.
 @pytest.mark.parametrize("B,T,H", [(1, 300, 7), (3, 700, 40), (2, 130, 64), (2, 300, 80), (1, 64, 129)])
 def test_two_kernel_entry_points(device, B, T, H):

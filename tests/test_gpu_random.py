@@ -90,7 +90,7 @@ def _packed_cases():
         lens = [rnd.choice([0, 1, 63, 64, 65]) if rnd.random() < 0.3 else rnd.randint(1, 300) for _ in range(n_seq)]
         if sum(lens) == 0:
             lens[0] = 5
-        big = i % 3 == 2                                   # one-kernel form (sequences * heads >= 96)
+        big = i % 3 == 2                                   # one-kernel form (sequences * heads >= 96, above the threshold of 72)
         H = rnd.randint(96 // n_seq + 1, 128 // n_seq + 8) if big else rnd.randint(1, max(1, 95 // n_seq))
         out.append((i, lens, H, rnd.choice(["model", "normal", "slow", "channels"]), rnd.random() < 0.7,
                     rnd.choice([0, 0, 7])))

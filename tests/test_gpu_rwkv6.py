@@ -49,7 +49,7 @@ def test_float32_matches_oracle(device, B, T, H):
     assert rel_l2(s, s_ref.transpose(-1, -2)) > 1e-2
 
 
-# B*H < 96: summaries + scan; B*H >= 96: the one-kernel form.  Ragged last chunks, one-token sequences of
+# B*H < 72: summaries + scan; B*H >= 72: the one-kernel form.  Ragged last chunks, one-token sequences of
 # chunks, long sequences.
 @pytest.mark.parametrize("B,T,H", [(1, 64, 1), (2, 200, 2), (4, 2, 8), (3, 65, 5), (1, 1024, 2),
                                    (4, 200, 32), (2, 130, 64), (5, 577, 40), (1, 200, 97)])

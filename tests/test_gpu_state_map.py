@@ -19,7 +19,7 @@ def _pool(n_state, H, seed):
     return 0.1 * torch.randn(n_state, H, 64, 64, generator=g)
 
 
-# fp32 recurrent path, two-kernel bf16 path (B*H < 96), fused bf16 path, T = 1 (decode kernel)
+# fp32 recurrent path, two-kernel bf16 path (B*H < 72), fused bf16 path, T = 1 (decode kernel)
 @pytest.mark.parametrize("B,T,H,dtype,tol", [(3, 70, 2, torch.float32, 1e-4), (3, 130, 4, torch.bfloat16, 5e-3),
                                              (4, 130, 32, torch.bfloat16, 5e-3), (5, 1, 3, torch.bfloat16, 5e-3)])
 def test_forward_with_state_map(device, B, T, H, dtype, tol):

@@ -64,7 +64,7 @@ def check_forward(device, lens, H, seed, with_h0=True, tail=0, cu_on_device=Fals
     return o, s, packed, parts, h0, cu
 
 
-# N*H < 96: summaries + scan (value-split scan); N*H >= 96: the one-kernel form; > 128 sequences*heads in
+# N*H < 72: summaries + scan (value-split scan); N*H >= 72: the one-kernel form; > 128 sequences*heads in
 # the two-kernel form cannot happen through rwkv7_fwd_varlen.  Lengths around the chunk size, a single
 # token, empty sequences first / in the middle / last, many short sequences.
 @pytest.mark.parametrize("lens,H", [
@@ -97,7 +97,7 @@ def test_varlen_forward_float32(device):
 
 
 def test_varlen_equals_separate_calls_bit_for_bit(device):
-    """Chunks are counted from each sequence's own first token, so below 96 sequence-heads (both calls
+    """Chunks are counted from each sequence's own first token, so below 72 sequence-heads (both calls
     take the summary + scan kernels) the packed call reproduces the per-sequence calls exactly."""
     lens, H = [70, 128, 30, 190, 64], 4          # (13 tokens or more: shorter dense calls take the recurrent kernel)
     packed, parts, h0, cu = pack(lens, H, seed=7300)
