@@ -158,8 +158,9 @@ __device__ __forceinline__ void state_load_wait(float4_t (&h)[4], uint32_t& car)
 // still shows its predecessor's field somewhere: two fields per 16-byte word catch a word torn at 8 bytes or
 // coarser (the memory system moves 32 bytes or more at a time).  A reader ahead of its turn may find an image
 // in the slot that is several uses old (with few heads the chip holds the workgroups of many chunk positions
-// at once); the 3-bit fields repeat every seven uses, the carrier's byte only every 255, which is further
-// than any reader can be ahead.
+// at once); the 3-bit fields repeat every seven uses, the carrier's byte every 255, the two together every
+// 1785 uses of a slot (3570 chunk positions), while a reader is at most as many positions ahead as the chip
+// holds workgroups (768).
 __device__ __forceinline__ uint32_t handoff_marks(unsigned long long tag, int c) {
     const uint32_t u = (uint32_t)(c >> 1);
     return ((1u + u % 7u) * 0x24924900u | (1u + u % 255u)) ^ (uint32_t)tag;
