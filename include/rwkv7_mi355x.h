@@ -42,8 +42,9 @@ extern "C" {
 #endif
 
 /* 2: the one-kernel forward's workspace holds a status record, two state slots per (batch, head) and their
- * carriers (sizes from the *_workspace_bytes functions as before); rwkv7_set_giveup_notice; RWKV6 float32 gradients */
-#define RWKV7_ABI_VERSION 2
+ * carriers (sizes from the *_workspace_bytes functions as before); rwkv7_set_giveup_notice; RWKV6 float32 gradients
+ * 3: the RWKV6 entry points take K = V = 128; rwkv6_bwd_workspace_bytes_head */
+#define RWKV7_ABI_VERSION 3
 
 /* element type of r, w, k, v, a, b, o and the input gradients */
 #define RWKV7_DTYPE_BF16 0

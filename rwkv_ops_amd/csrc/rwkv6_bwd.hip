@@ -19,8 +19,8 @@ namespace rwkv7 {
 
 namespace {
 
-// cu[2b] = b*T, cu[2b+1] = b*T + T-1 (b < B), which ends at B*T - 1; and a zero-filled [B*T, H, 64] bf16
-// tensor to stand for a and b
+// cu[2b] = b*T, cu[2b+1] = b*T + T-1 (b < B), which ends at B*T - 1; and a zero-filled [B*T, H, N] tensor
+// to stand for a and b
 __global__ __launch_bounds__(256)
 void rwkv6_bwd_prologue_kernel(int* __restrict__ cu, u32x4_t* __restrict__ zeros, int64_t n16, int B, int T)
 {
@@ -30,13 +30,14 @@ void rwkv6_bwd_prologue_kernel(int* __restrict__ cu, u32x4_t* __restrict__ zeros
     for (int64_t i = i0; i < n16; i += (int64_t)gridDim.x * 256) zeros[i] = z;
 }
 
-// One workgroup per (batch, head, 64 tokens), lane = channel, wave v takes tokens v, v+4, ...:
+// One workgroup per (batch, head, 64 tokens), lane = channel (N = 128: channels lane and lane + 64), wave v takes
+// tokens v, v+4, ...:
 //   s = <dy_t, v_t>, q = sum_c r u k;
 //   dr_t = dr'_{t-1} + u k s,  dk_t = dk'_t + u r s,  dv_t = dv'_t + q dy_t,  dw_t = dw'_t,
 // the primed terms being zero where the state path has none (t = 0 for dr, t = T-1 for the others; the
 // buffers hold the dummy sequences' values or nothing there).  dk, dv, dw are corrected in place.
 // du[h][c] = sum over batch and tokens of r k s: summed per workgroup, then one atomic per channel.
-template <typename E>
+template <typename E, int N>
 __global__ __launch_bounds__(256)
 void rwkv6_bwd_epilogue_kernel(const E* __restrict__ r, const E* __restrict__ k,
                                const E* __restrict__ v, const E* __restrict__ u,
@@ -44,33 +45,49 @@ void rwkv6_bwd_epilogue_kernel(const E* __restrict__ r, const E* __restrict__ k,
                                E* __restrict__ dr, E* __restrict__ dk, E* __restrict__ dv,
                                E* __restrict__ dw, float* __restrict__ du, int T, int H, int state_path)
 {
-    __shared__ float part[4][HEAD];
+    constexpr int PER = N / 64;                  // channels per lane
+    __shared__ float part[4][N];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int nblk = (T + 63) / 64;
     const int blk = blockIdx.x % nblk, hi = (blockIdx.x / nblk) % H, bi = blockIdx.x / (nblk * H);
-    const float uc = (float)u[hi * HEAD + lane];
-    float du_acc = 0.f;
+    float uc[PER], du_acc[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) { uc[j] = (float)u[hi * N + lane + 64 * j]; du_acc[j] = 0.f; }
     for (int tt = wv; tt < 64; tt += 4) {
         const int t = blk * 64 + tt;
         if (t >= T) break;
-        const int64_t row = (((int64_t)bi * T + t) * H + hi) * HEAD + lane;
-        const float rc = (float)r[row], kc = (float)k[row], vc = (float)v[row], gc = (float)dy[row];
-        float s = gc * vc, q = rc * uc * kc;
+        const int64_t row0 = (((int64_t)bi * T + t) * H + hi) * N + lane;
+        float rc[PER], kc[PER], vc[PER], gc[PER];
+        float s = 0.f, q = 0.f;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int64_t row = row0 + 64 * j;
+            rc[j] = (float)r[row]; kc[j] = (float)k[row]; vc[j] = (float)v[row]; gc[j] = (float)dy[row];
+            s = fmaf(gc[j], vc[j], s);
+            q = fmaf(rc[j] * uc[j], kc[j], q);
+        }
 #pragma unroll
         for (int m = 32; m >= 1; m >>= 1) { s += __shfl_xor(s, m, 64); q += __shfl_xor(q, m, 64); }
         const bool first = t == 0, last = t == T - 1;
-        const float dr0 = (state_path && !first) ? (float)dr_state[row - (int64_t)H * HEAD] : 0.f;
-        const float dk0 = (state_path && !last) ? (float)dk[row] : 0.f;
-        const float dv0 = (state_path && !last) ? (float)dv[row] : 0.f;
-        dr[row] = (E)(dr0 + uc * kc * s);
-        dk[row] = (E)(dk0 + uc * rc * s);
-        dv[row] = (E)(dv0 + q * gc);
-        if (!state_path || last) dw[row] = (E)0.f;
-        du_acc = fmaf(rc * kc, s, du_acc);
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int64_t row = row0 + 64 * j;
+            const float dr0 = (state_path && !first) ? (float)dr_state[row - (int64_t)H * N] : 0.f;
+            const float dk0 = (state_path && !last) ? (float)dk[row] : 0.f;
+            const float dv0 = (state_path && !last) ? (float)dv[row] : 0.f;
+            dr[row] = (E)(dr0 + uc[j] * kc[j] * s);
+            dk[row] = (E)(dk0 + uc[j] * rc[j] * s);
+            dv[row] = (E)(dv0 + q * gc[j]);
+            if (!state_path || last) dw[row] = (E)0.f;
+            du_acc[j] = fmaf(rc[j] * kc[j], s, du_acc[j]);
+        }
     }
-    part[wv][lane] = du_acc;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) part[wv][lane + 64 * j] = du_acc[j];
     __syncthreads();
-    if (wv == 0) atomicAdd(du + hi * HEAD + lane, part[0][lane] + part[1][lane] + part[2][lane] + part[3][lane]);
+    if (threadIdx.x < N)
+        atomicAdd(du + hi * N + threadIdx.x,
+                  part[0][threadIdx.x] + part[1][threadIdx.x] + part[2][threadIdx.x] + part[3][threadIdx.x]);
 }
 
 __global__ void rwkv6_zero_du_kernel(float* du, int n) {
@@ -83,31 +100,44 @@ size_t align256(size_t x) { return (x + 255) / 256 * 256; }
 }  // namespace
 
 // workspace: [cu table][zeros][dr of the state path][da, db dump][RWKV7 backward workspace]
-size_t rwkv6_bwd_workspace_bytes(int B, int T, int H, int dtype) {
+// (N = 128: the state path is the float32 recurrent backward over the same table, as for RWKV7 at that head size)
+size_t rwkv6_bwd_workspace_bytes(int B, int T, int H, int N, int dtype) {
     const bool f32 = dtype == RWKV7_DTYPE_F32;
-    const size_t tensor = align256((size_t)B * T * H * HEAD * (f32 ? 4 : 2));
+    const size_t tensor = align256((size_t)B * T * H * N * (f32 ? 4 : 2));
     size_t n = align256((size_t)2 * B * 4) + 3 * tensor;
-    if (T > 1) n += f32 ? bwd_chunk_f32_workspace_bytes(2 * B - 1, B * T - 1, H, true)
-                        : bwd_chunk_workspace_bytes(2 * B - 1, B * T - 1, H, true);
+    if (T > 1) n += N == 128 ? bwd_recurrent_workspace_bytes(2 * B - 1, B * T - 1, H, 128, true)
+                  : f32      ? bwd_chunk_f32_workspace_bytes(2 * B - 1, B * T - 1, H, true)
+                             : bwd_chunk_workspace_bytes(2 * B - 1, B * T - 1, H, true);
     return n;
+}
+
+template <typename E, int N>
+static void launch_epilogue(const void* r, const void* k, const void* v, const void* u, const void* dy,
+                            const void* dr_state, void* dr, void* dk, void* dv, void* dw, float* du,
+                            int B, int T, int H, hipStream_t stream)
+{
+    const int nblk = (T + 63) / 64;
+    rwkv6_bwd_epilogue_kernel<E, N><<<dim3((unsigned)(B * H * nblk)), dim3(256), 0, stream>>>(
+        (const E*)r, (const E*)k, (const E*)v, (const E*)u, (const E*)dy, (const E*)dr_state,
+        (E*)dr, (E*)dk, (E*)dv, (E*)dw, du, T, H, T > 1 ? 1 : 0);
 }
 
 hipError_t launch_rwkv6_bwd(const void* r, const void* k, const void* v, const void* w, const void* u,
                             const void* dy, void* dr, void* dk, void* dv, void* dw, float* du,
-                            int B, int T, int H, int dtype, void* ws, hipStream_t stream)
+                            int B, int T, int H, int N, int dtype, void* ws, hipStream_t stream)
 {
     // float32 tensors: the same plan on the chunked float32 backward (every product on the float32 matrix cores),
     // so that float32 callers get float32 gradients as the reference's float32 kernel gives them
     // (/root/reference/rwkv_ops/rwkv6_kernel/torch_rwkv_kernel.py:137)
     const bool f32 = dtype == RWKV7_DTYPE_F32;
-    const size_t tensor = align256((size_t)B * T * H * HEAD * (f32 ? 4 : 2));
+    const size_t tensor = align256((size_t)B * T * H * N * (f32 ? 4 : 2));
     unsigned char* base = static_cast<unsigned char*>(ws);
     int* cu = reinterpret_cast<int*>(base);
     unsigned char* zeros = base + align256((size_t)2 * B * 4);
     unsigned char* dr_state = zeros + tensor;
     unsigned char* dump = dr_state + tensor;
     void* bws = dump + tensor;
-    rwkv6_zero_du_kernel<<<dim3((unsigned)((H * HEAD + 255) / 256)), dim3(256), 0, stream>>>(du, H * HEAD);
+    rwkv6_zero_du_kernel<<<dim3((unsigned)((H * N + 255) / 256)), dim3(256), 0, stream>>>(du, H * N);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (T > 1) {
@@ -117,25 +147,24 @@ hipError_t launch_rwkv6_bwd(const void* r, const void* k, const void* v, const v
             cu, reinterpret_cast<u32x4_t*>(zeros), n16, B, T);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
-        const int64_t ahead = (int64_t)H * HEAD * (f32 ? 4 : 2);          // one token, in bytes
+        const int64_t ahead = (int64_t)H * N * (f32 ? 4 : 2);             // one token, in bytes
         BwdArgs p;
         p.r = static_cast<const unsigned char*>(r) + ahead; p.w = w; p.k = k; p.v = v; p.a = zeros; p.b = zeros;
         p.h0 = nullptr; p.h0_batch_stride = 0;
         p.dO = static_cast<const unsigned char*>(dy) + ahead; p.dht = nullptr;
         p.dr = dr_state; p.dw = dw; p.dk = dk; p.dv = dv; p.da = dump; p.db = dump; p.dh0 = nullptr;
         p.B = 2 * B - 1; p.T = B * T - 1; p.H = H; p.dtype = dtype; p.cu = cu;
-        e = f32 ? launch_bwd_chunk_f32(p, bws, stream) : launch_bwd_chunk(p, bws, stream);
+        e = N == 128 ? launch_bwd_recurrent(p, 128, bws, stream)
+            : f32    ? launch_bwd_chunk_f32(p, bws, stream) : launch_bwd_chunk(p, bws, stream);
         if (e != hipSuccess) return e;
     }
-    const int nblk = (T + 63) / 64;
-    if (f32)
-        rwkv6_bwd_epilogue_kernel<float><<<dim3((unsigned)(B * H * nblk)), dim3(256), 0, stream>>>(
-            (const float*)r, (const float*)k, (const float*)v, (const float*)u, (const float*)dy,
-            (const float*)dr_state, (float*)dr, (float*)dk, (float*)dv, (float*)dw, du, T, H, T > 1 ? 1 : 0);
-    else
-        rwkv6_bwd_epilogue_kernel<bf16_t><<<dim3((unsigned)(B * H * nblk)), dim3(256), 0, stream>>>(
-            (const bf16_t*)r, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)u, (const bf16_t*)dy,
-            (const bf16_t*)dr_state, (bf16_t*)dr, (bf16_t*)dk, (bf16_t*)dv, (bf16_t*)dw, du, T, H, T > 1 ? 1 : 0);
+    if (N == 128) {
+        if (f32) launch_epilogue<float, 128>(r, k, v, u, dy, dr_state, dr, dk, dv, dw, du, B, T, H, stream);
+        else launch_epilogue<bf16_t, 128>(r, k, v, u, dy, dr_state, dr, dk, dv, dw, du, B, T, H, stream);
+    } else {
+        if (f32) launch_epilogue<float, HEAD>(r, k, v, u, dy, dr_state, dr, dk, dv, dw, du, B, T, H, stream);
+        else launch_epilogue<bf16_t, HEAD>(r, k, v, u, dy, dr_state, dr, dk, dv, dw, du, B, T, H, stream);
+    }
     return hipGetLastError();
 }
 

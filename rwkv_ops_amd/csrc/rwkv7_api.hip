@@ -59,7 +59,7 @@ const char* rwkv7_status_string(int status) {
         case RWKV7_OK: return "ok";
         case RWKV7_ERR_NULL_POINTER: return "a required pointer is NULL";
         case RWKV7_ERR_BAD_DTYPE: return "dtype must be RWKV7_DTYPE_BF16 (0), RWKV7_DTYPE_F32 (1) or RWKV7_DTYPE_F16 (2)";
-        case RWKV7_ERR_BAD_HEAD_SIZE: return "K = V = 64 (every entry point) or 128 (every entry point but the two-kernel ones and the RWKV6 operator) only";
+        case RWKV7_ERR_BAD_HEAD_SIZE: return "K = V = 64 (every entry point) or 128 (every entry point but the two-kernel ones) only";
         case RWKV7_ERR_BAD_SHAPE: return "B, T and H must be >= 1 and B*H*ceil(T/64) <= 2^30";
         case RWKV7_ERR_BAD_STRIDE: return "h0_batch_stride must be 0 (broadcast) or H*K*V";
         case RWKV7_ERR_WORKSPACE: return "workspace is NULL, not 256-byte aligned or too small";
@@ -482,7 +482,7 @@ int pack_rwkv6(const void* r, const void* k, const void* v, const void* w, const
                int B, int T, int H, int K, int V, int dtype, SeqArgs& p)
 {
     // a and b do not exist for this operator: r stands in for them in the common checks
-    int rc = check_seq(r, w, k, v, r, r, states, (int64_t)H * 64 * 64, y, ys, B, T, H, K, V, dtype);
+    int rc = check_seq(r, w, k, v, r, r, states, (int64_t)H * K * V, y, ys, B, T, H, K, V, dtype, true);
     if (rc != RWKV7_OK) return rc;
     if (!u) return RWKV7_ERR_NULL_POINTER;
     if (!aligned16(u) || (reinterpret_cast<uintptr_t>(state_map) & 3u) != 0) return RWKV7_ERR_ALIGNMENT;
@@ -493,7 +493,7 @@ int pack_rwkv6(const void* r, const void* k, const void* v, const void* w, const
         return RWKV7_ERR_NULL_POINTER;
     }
     p = pack(r, w, k, v, nullptr, nullptr, states,
-             (states && !state_map && n_state == 1 && B != 1) ? 0 : (int64_t)H * 64 * 64, y, ys, B, T, H, dtype);
+             (states && !state_map && n_state == 1 && B != 1) ? 0 : (int64_t)H * K * V, y, ys, B, T, H, dtype, K);
     p.u6 = u;
     if (states && state_map) { p.h0_map = state_map; p.n_state = n_state; }
     return RWKV7_OK;
@@ -512,7 +512,7 @@ int rwkv6_fwd(const void* r, const void* k, const void* v, const void* w, const 
     int rc = pack_rwkv6(r, k, v, w, u, states, n_state, state_map, y, ys, B, T, H, K, V, dtype, p);
     if (rc != RWKV7_OK) return rc;
     if (T == 1) return (int)rwkv7::launch_decode(p, static_cast<hipStream_t>(stream));
-    if (dtype == RWKV7_DTYPE_F32 || T <= RECURRENT_MAX_T)
+    if (dtype == RWKV7_DTYPE_F32 || T <= RECURRENT_MAX_T || K == 128)
         return (int)rwkv7::launch_rwkv6_recurrent(p, static_cast<hipStream_t>(stream));
     const size_t need = rwkv6_fwd_workspace_bytes(B, T, H, dtype);
     if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return RWKV7_ERR_WORKSPACE;
@@ -530,9 +530,14 @@ int rwkv6_fwd_recurrent(const void* r, const void* k, const void* v, const void*
     return (int)rwkv7::launch_rwkv6_recurrent(p, static_cast<hipStream_t>(stream));
 }
 
+size_t rwkv6_bwd_workspace_bytes_head(int B, int T, int H, int K, int dtype) {
+    if ((dtype != RWKV7_DTYPE_BF16 && dtype != RWKV7_DTYPE_F32) || B < 1 || T < 1 || H < 1 || (K != 64 && K != 128))
+        return 0;
+    return rwkv7::rwkv6_bwd_workspace_bytes(B, T, H, K, dtype);
+}
+
 size_t rwkv6_bwd_workspace_bytes(int B, int T, int H, int dtype) {
-    if ((dtype != RWKV7_DTYPE_BF16 && dtype != RWKV7_DTYPE_F32) || B < 1 || T < 1 || H < 1) return 0;
-    return rwkv7::rwkv6_bwd_workspace_bytes(B, T, H, dtype);
+    return rwkv6_bwd_workspace_bytes_head(B, T, H, 64, dtype);
 }
 
 int rwkv6_bwd(const void* r, const void* k, const void* v, const void* w, const void* u, const void* d_y,
@@ -540,16 +545,16 @@ int rwkv6_bwd(const void* r, const void* k, const void* v, const void* w, const 
               int B, int T, int H, int K, int V, int dtype, void* ws, size_t ws_bytes, void* stream)
 {
     if (dtype == RWKV7_DTYPE_F16) return RWKV7_ERR_UNSUPPORTED;
-    int rc = check_seq(r, w, k, v, r, r, nullptr, 0, dr, nullptr, B, T, H, K, V, dtype);
+    int rc = check_seq(r, w, k, v, r, r, nullptr, 0, dr, nullptr, B, T, H, K, V, dtype, true);
     if (rc != RWKV7_OK) return rc;
     // the state path runs as 2B - 1 packed sequences over B*T - 1 tokens
     if ((((int64_t)B * T) >> 6) + 2 * (int64_t)B > ((int64_t)1 << 30) / H) return RWKV7_ERR_BAD_SHAPE;
     if (!u || !d_y || !dk || !dv || !dw || !du) return RWKV7_ERR_NULL_POINTER;
     if (!aligned16(u) || !aligned16(d_y) || !aligned16(dk) || !aligned16(dv) || !aligned16(dw) || !aligned16(du))
         return RWKV7_ERR_ALIGNMENT;
-    const size_t need = rwkv7::rwkv6_bwd_workspace_bytes(B, T, H, dtype);
+    const size_t need = rwkv7::rwkv6_bwd_workspace_bytes(B, T, H, K, dtype);
     if (!ws || ws_bytes < need || (reinterpret_cast<uintptr_t>(ws) & 255u) != 0) return RWKV7_ERR_WORKSPACE;
-    return (int)rwkv7::launch_rwkv6_bwd(r, k, v, w, u, d_y, dr, dk, dv, dw, du, B, T, H, dtype, ws,
+    return (int)rwkv7::launch_rwkv6_bwd(r, k, v, w, u, d_y, dr, dk, dv, dw, du, B, T, H, K, dtype, ws,
                                         static_cast<hipStream_t>(stream));
 }
 

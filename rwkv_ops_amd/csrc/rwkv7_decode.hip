@@ -112,7 +112,14 @@ template <typename T>
 static hipError_t launch_decode_t(const SeqArgs& p, hipStream_t stream) {
     const int64_t units = (p.N / 32) * (int64_t)p.B * p.H;
     const unsigned grid = (unsigned)((units + DECODE_WAVES - 1) / DECODE_WAVES);
-    if (p.N == 128) {                 // RWKV7 only
+    if (p.N == 128 && p.u6 != nullptr) {
+        decode_kernel<T, true, true, true, 128><<<dim3(grid), dim3(64 * DECODE_WAVES), 0, stream>>>(
+            (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, nullptr, (const T*)p.u6,
+            p.h0, p.h0_batch_stride, p.h0_map, p.n_state, (T*)p.o, p.ht_in_place ? const_cast<float*>(p.h0) : p.ht,
+            p.ht_in_place ? 1 : 0, p.B, p.H);
+        return hipGetLastError();
+    }
+    if (p.N == 128) {
         decode_kernel<T, true, true, false, 128><<<dim3(grid), dim3(64 * DECODE_WAVES), 0, stream>>>(
             (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, (const T*)p.a, (const T*)p.b,
             p.h0, p.h0_batch_stride, p.h0_map, p.n_state, (T*)p.o, p.ht_in_place ? const_cast<float*>(p.h0) : p.ht,

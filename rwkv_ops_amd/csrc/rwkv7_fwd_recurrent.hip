@@ -245,16 +245,18 @@ hipError_t launch_fwd_recurrent_states(const SeqArgs& p, float* states, int seg,
                                         : launch_states_t<float, 64>(p, states, seg, stream);
 }
 
-template <typename T>
+template <typename T, int N>
 static hipError_t launch6_t(const SeqArgs& p, hipStream_t stream) {
-    fwd_recurrent_kernel<T, HEAD, true><<<dim3((unsigned)(p.B * p.H)), dim3(256), 0, stream>>>(
+    fwd_recurrent_kernel<T, N, true><<<dim3((unsigned)(p.B * p.H)), dim3(256), 0, stream>>>(
         (const T*)p.r, (const T*)p.w, (const T*)p.k, (const T*)p.v, nullptr, (const T*)p.u6,
         p.h0, p.h0_batch_stride, p.h0_map, p.n_state, (T*)p.o, p.ht, seq_layout(p, nullptr));
     return hipGetLastError();
 }
 
 hipError_t launch_rwkv6_recurrent(const SeqArgs& p, hipStream_t stream) {
-    return p.dtype == RWKV7_DTYPE_BF16 ? launch6_t<bf16_t>(p, stream) : launch6_t<float>(p, stream);
+    if (p.N == 128)
+        return p.dtype == RWKV7_DTYPE_BF16 ? launch6_t<bf16_t, 128>(p, stream) : launch6_t<float, 128>(p, stream);
+    return p.dtype == RWKV7_DTYPE_BF16 ? launch6_t<bf16_t, HEAD>(p, stream) : launch6_t<float, HEAD>(p, stream);
 }
 
 hipError_t launch_fwd_recurrent(const SeqArgs& p, hipStream_t stream) {

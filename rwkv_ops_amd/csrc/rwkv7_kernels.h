@@ -106,10 +106,10 @@ size_t bwd_chunk_f32_workspace_bytes(int B, int T, int H, bool varlen = false);
 hipError_t launch_bwd_chunk_f32(const BwdArgs& p, void* ws, hipStream_t stream);
 // RWKV6 backward (stateless call, bf16 or float32): runs the RWKV7 backward kernels on operands read one token ahead
 // plus an epilogue for the bonus term; du is float32 [H, 64]
-size_t rwkv6_bwd_workspace_bytes(int B, int T, int H, int dtype);
+size_t rwkv6_bwd_workspace_bytes(int B, int T, int H, int N, int dtype);
 hipError_t launch_rwkv6_bwd(const void* r, const void* k, const void* v, const void* w, const void* u,
                             const void* dy, void* dr, void* dk, void* dv, void* dw, float* du,
-                            int B, int T, int H, int dtype, void* ws, hipStream_t stream);
+                            int B, int T, int H, int N, int dtype, void* ws, hipStream_t stream);
 // the backward's variant of the chunk summaries (rwkv7_fwd_chunk.hip)
 hipError_t launch_bwd_summary(const SeqArgs& p, const SeqLayout& L, const void* d_o, void* qdo, void* pp,
                               void* qc, float* eg, hipStream_t stream);

@@ -35,21 +35,21 @@ from ..rwkv7.op import _as_state_map, _dtype_code, _on_device, _ptr, _require_gp
 
 __all__ = ["RWKVKernelOperator", "get_rwkv6_kernel"]
 
-HEAD_SIZE = 64
+HEAD_SIZES = (64, 128)
 
 
-def _forward(xs, states, n_state, smap, with_state, B, T, H, dt):
+def _forward(xs, states, n_state, smap, with_state, B, T, H, N, dt):
     """One rwkv6_fwd call: ``xs`` = (r, k, v, w, u) contiguous in ``dt``; returns (y, final states or None)."""
     code = _dtype_code(dt)
     lib = _lib.load()
     dev = xs[0].device
-    y = torch.empty((B, T, H * HEAD_SIZE), dtype=dt, device=dev)
-    ys = torch.empty((B, H, HEAD_SIZE, HEAD_SIZE), dtype=torch.float32, device=dev) if with_state else None
+    y = torch.empty((B, T, H * N), dtype=dt, device=dev)
+    ys = torch.empty((B, H, N, N), dtype=torch.float32, device=dev) if with_state else None
     with _on_device(dev):
-        ws_bytes = lib.rwkv6_fwd_workspace_bytes(B, T, H, code)
+        ws_bytes = lib.rwkv6_fwd_workspace_bytes(B, T, H, code) if N == 64 else 0     # head size 128: no workspace
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
         rc = lib.rwkv6_fwd(*[_ptr(x) for x in xs], _ptr(states), n_state, _ptr(smap), _ptr(y), _ptr(ys),
-                           B, T, H, HEAD_SIZE, HEAD_SIZE, code, _ptr(ws), ws_bytes, _stream_ptr(dev))
+                           B, T, H, N, N, code, _ptr(ws), ws_bytes, _stream_ptr(dev))
     _lib.check(rc, "rwkv6_fwd")
     return y, ys
 
@@ -68,7 +68,7 @@ class _Rwkv6Function(torch.autograd.Function):
     @staticmethod
     def forward(ctx, r, k, v, w, u, H):
         B, T, _ = r.shape
-        y, _ = _forward((r, k, v, w, u), None, 0, None, False, B, T, H, r.dtype)
+        y, _ = _forward((r, k, v, w, u), None, 0, None, False, B, T, H, r.shape[2] // H, r.dtype)
         ctx.save_for_backward(r, k, v, w, u)
         ctx.H = H
         return y
@@ -78,18 +78,18 @@ class _Rwkv6Function(torch.autograd.Function):
         r, k, v, w, u = ctx.saved_tensors
         B, T, C = r.shape
         H = ctx.H
+        N = C // H
         dt = r.dtype                       # bfloat16 or float32: the kernels of that type (float32 gradients for
         code = _dtype_code(dt)             # float32 tensors, torch_rwkv_kernel.py:137)
         g = gy.to(dt).contiguous()
         lib = _lib.load()
         grads = [torch.empty((B, T, C), dtype=dt, device=r.device) for _ in range(4)]
-        du = torch.empty((H, HEAD_SIZE), dtype=torch.float32, device=r.device)
+        du = torch.empty((H, N), dtype=torch.float32, device=r.device)
         with _on_device(r.device):
-            ws_bytes = lib.rwkv6_bwd_workspace_bytes(B, T, H, code)
+            ws_bytes = lib.rwkv6_bwd_workspace_bytes_head(B, T, H, N, code)
             ws = torch.empty(ws_bytes, dtype=torch.uint8, device=r.device)
             rc = lib.rwkv6_bwd(*[_ptr(x) for x in (r, k, v, w, u)], _ptr(g), *[_ptr(x) for x in grads], _ptr(du),
-                               B, T, H, HEAD_SIZE, HEAD_SIZE, code, _ptr(ws), ws_bytes,
-                               _stream_ptr(r.device))
+                               B, T, H, N, N, code, _ptr(ws), ws_bytes, _stream_ptr(r.device))
         _lib.check(rc, "rwkv6_bwd")
         dr, dk, dv, dw = (x.to(dt) for x in grads)
         return dr, dk, dv, dw, du.reshape(u.shape).to(u.dtype), None
@@ -98,9 +98,10 @@ class _Rwkv6Function(torch.autograd.Function):
 class RWKVKernelOperator:
     def __init__(self, head_size: int, max_sequence_length: Optional[int] = None,
                  state_dtype: Optional[torch.dtype] = None):
-        if int(head_size) != HEAD_SIZE:
-            raise NotImplementedError(f"head_size={head_size}: only a head size of {HEAD_SIZE} is built")
-        self.head_size = HEAD_SIZE
+        if int(head_size) not in HEAD_SIZES:
+            # (the reference compiles its kernels for the head size it is given, torch_rwkv_kernel.py:22-45)
+            raise NotImplementedError(f"head_size={head_size}: head sizes {HEAD_SIZES} are built")
+        self.head_size = int(head_size)
         self.max_sequence_length = max_sequence_length      # the kernels have no length limit
         self.state_dtype = state_dtype
 
@@ -159,7 +160,7 @@ class RWKVKernelOperator:
         xs = [x if (x.dtype == dt and x.is_contiguous()) else x.to(dt).contiguous() for x in (r, k, v, w, u)]
         if needs_grad:
             return _Rwkv6Function.apply(*xs, H).to(out_dtype), None
-        y, ys = _forward(xs, states, n_state, smap, with_state, B, T, H, dt)
+        y, ys = _forward(xs, states, n_state, smap, with_state, B, T, H, self.head_size, dt)
         y = y.to(out_dtype)
         if not with_state:
             return y, None

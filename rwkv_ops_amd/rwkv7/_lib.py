@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(_CSRC, "librwkv7_mi355x.so")
 DTYPE_BF16, DTYPE_F32, DTYPE_F16 = 0, 1, 2
 NO_STATUS_RECORD = ctypes.c_size_t(-1).value
 FWD_DONE, FWD_GAVE_UP, FWD_NO_LAUNCH = 0, 1, 2
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _P, _I, _I64, _SZ = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64, ctypes.c_size_t
 
@@ -47,6 +47,7 @@ SIGNATURES = {
     "rwkv6_fwd_workspace_bytes": (_SZ, [_I, _I, _I, _I]),
     "rwkv6_fwd": (_I, [_P] * 5 + [_P, _I, _P, _P, _P] + [_I] * 6 + [_P, _SZ, _P]),
     "rwkv6_bwd_workspace_bytes": (_SZ, [_I, _I, _I, _I]),
+    "rwkv6_bwd_workspace_bytes_head": (_SZ, [_I, _I, _I, _I, _I]),
     "rwkv6_bwd": (_I, [_P] * 6 + [_P] * 5 + [_I] * 6 + [_P, _SZ, _P]),
     "rwkv6_fwd_recurrent": (_I, [_P] * 5 + [_P, _I, _P, _P, _P] + [_I] * 6 + [_P]),
     "rwkv7_fwd_recurrent": (_I, [_P] * 6 + [_P, _I64, _P, _P] + [_I] * 6 + [_P]),

@@ -140,6 +140,12 @@ def test_rwkv6_argument_errors_do_not_launch():
     assert lib.rwkv6_bwd_workspace_bytes(2, 8, 2, 0) > 3 * 2 * 8 * 2 * 64 * 2
     assert lib.rwkv6_bwd_workspace_bytes(2, 8, 2, 1) > 3 * 2 * 8 * 2 * 64 * 4
     assert lib.rwkv6_bwd_workspace_bytes(2, 8, 2, 2) == 0
+    # the head size as an argument: 64 is the plain function, 128 is built (larger tensors), others are not
+    assert lib.rwkv6_bwd_workspace_bytes_head(2, 8, 2, 64, 0) == lib.rwkv6_bwd_workspace_bytes(2, 8, 2, 0)
+    assert lib.rwkv6_bwd_workspace_bytes_head(2, 8, 2, 128, 0) > 3 * 2 * 8 * 2 * 128 * 2
+    assert lib.rwkv6_bwd_workspace_bytes_head(2, 8, 2, 128, 1) > 3 * 2 * 8 * 2 * 128 * 4
+    assert lib.rwkv6_bwd_workspace_bytes_head(2, 8, 2, 96, 0) == 0
+    assert fwd(K=128) == -3                              # K = 128 against V = 64
 
 
 def test_float16_is_a_dtype_only_where_a_kernel_reads_it():

@@ -127,7 +127,7 @@ def test_dtype_conventions(device):
     with pytest.raises(NotImplementedError):                               # gradients: the stateless call only
         op(leaf, *[x.to(device) for x in xs[1:5]], with_state=True)
     with pytest.raises(NotImplementedError):
-        rwkv_ops_amd.RWKV6_OP(128, 128)
+        rwkv_ops_amd.RWKV6_OP(96, 128)
 
 
 # The bf16 chunked formulation costs the RWKV7 gradients 3e-3 .. 6e-3 relative L2 (tests/test_gpu_backward.py);
