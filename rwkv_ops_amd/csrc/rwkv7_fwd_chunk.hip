@@ -63,6 +63,7 @@ constexpr int OFF_DO = 24576;          //   then (backward) the dO tile
 constexpr int OFF_FQ = 24576;          //   then (fused) the exchanged halves of Qt
 constexpr int OFF_AQK = 32768;         // 6 sigma fragments of Aqk [i][j]                                  Bx .. Bf1
 constexpr int OFF_AQB = 38912;
+constexpr int OFF_QG_P2 = 32768;       //   before them (one bucket): a copy of the qg tile for the waves that take other rows' blocks  B1 .. Bx
 constexpr int OFF_OT = 32768;          //   then (fused) the O tile, transposed
 constexpr int OFF_AAB = 45056;         // the 6 blocks of Aab below the diagonal, 16x16 bf16 row-major [i][j] (512 B each)
 constexpr int OFF_DI = 48128;          // 4 inverted diagonal blocks, bf16, row-major (512 B each)
@@ -439,6 +440,7 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
         const int at = tile_at(t_local, 32 * s + 8 * g);
         *reinterpret_cast<bf16x8_t*>(smem + OFF_AG + at) = AG[s];
         *reinterpret_cast<bf16x8_t*>(smem + OFF_V + at) = V[s];
+        if constexpr (SINGLE) *reinterpret_cast<bf16x8_t*>(smem + OFF_QG_P2 + at) = QG[s];
     }
     __syncthreads();                                                           // B1
 
@@ -448,106 +450,173 @@ void chunk_summary_kernel(const bf16_t* __restrict__ r_, const bf16_t* __restric
     bf16x8_t Vtr[2];
     Vtr[0] = tile_read_tr_frag(smem, OFF_V, w, 0, lane);
     Vtr[1] = tile_read_tr_frag(smem, OFF_V, w, 1, lane);
-    float4_t acc_qk[4], acc_qb[4], acc_ak[4], acc_ab[4];
     float4_t diagX = zero4;                 // D layout of X = Aab[w][w] (rows i, column j)
+    float4_t diagXT = zero4;                // D layout of X^T (rows j, column i)
+    if constexpr (SINGLE) {
+        // One bucket: the ten blocks (I, J), J <= I, of the four matrices are dealt out evenly instead of by rows
+        // (by rows wave 3 has four blocks and wave 0 one, and wave w of every workgroup of a CU sits on SIMD w):
+        // a wave takes the diagonal block of its own row and the one left of it; of the three blocks that leaves,
+        // wave 0 takes (3, 0) and (3, 1), wave 1 takes (2, 0).  A block of another row reads that row's qg / ag
+        // from the tiles (qg has a copy there for this phase); k~, b~ come from their fragments as before.
+        struct Set { float4_t qk, qb, ak, ab; };
+        auto clear = [&](Set& a) { a.qk = zero4; a.qb = zero4; a.ak = zero4; a.ab = zero4; };
+        auto block = [&](Set& a, int J, const bf16x8_t (&Q)[2], const bf16x8_t (&A_)[2]) {
 #pragma unroll
-    for (int J = 0; J < 4; ++J) {           // tiles right of the diagonal block (J > w) are never touched
-        if (J <= w) { acc_qk[J] = zero4; acc_qb[J] = zero4; acc_ak[J] = zero4; acc_ab[J] = zero4; }
-    }
-    bf16x8_t Qp[2] = {QG[0], QG[1]}, Ap[2] = {AG[0], AG[1]};
-    for (int p = 0; p < np; ++p) {
-        if constexpr (!SINGLE) {
-            if (p > 0) {                    // rare: tokens whose cumulative decay lies in bucket p
-                __syncthreads();
-                const float base = BUCKET * (float)p;
-                float xs2[16], X2[16];
-                bf16x8_t W2[2], R2[2], K2[2], A2[2], B2[2];
-                int lane_o = lane;
-                asm volatile("" : "+v"(lane_o));
-                const int64_t at = first_piece(lane_o);
-                load2(w_, at, W2); load2(r_, at, R2); load2(k_, at, K2);
-                if constexpr (V6) {
-                    A2[0] = A2[1] = B2[0] = B2[1] = load_frag_global(nullptr, false);
-                } else {
-                    load2(a_, at, A2); load2(b_, at, B2);
+            for (int s = 0; s < 2; ++s) {
+                const bf16x8_t kt = lds_read_frag(smem, OFF_KT, J * 2 + s, lane);
+                const bf16x8_t bt = lds_read_frag(smem, OFF_BT, J * 2 + s, lane);
+                a.qk = mfma_bf16(kt, Q[s], a.qk);
+                if constexpr (!V6) {           // RWKV6: a = b = 0, these three stay zero
+                    a.qb = mfma_bf16(bt, Q[s], a.qb);
+                    a.ak = mfma_bf16(kt, A_[s], a.ak);
+                    a.ab = mfma_bf16(bt, A_[s], a.ab);
                 }
-                if (ragged) {
-                    asm volatile("" ::: "memory");
-                    if (!valid) R2[0] = R2[1] = K2[0] = K2[1] = A2[0] = A2[1] = B2[0] = B2[1] = load_frag_global(nullptr, false);
-                }
-                decays(W2, xs2, X2);
-                add_prefix(X2);
-                float rf[16], kf[16], af[16], bf_[16];
-                unpack8(R2[0], rf); unpack8(R2[1], rf + 8); unpack8(K2[0], kf); unpack8(K2[1], kf + 8);
-                unpack8(A2[0], af); unpack8(A2[1], af + 8); unpack8(B2[0], bf_); unpack8(B2[1], bf_ + 8);
-#pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const float xi = X2[e], xe = xi - xs2[e];        // xe: up to, not including, this token
-                    const float up = (xi >= base && xi < base + BUCKET) ? ex2(xi - base) : 0.f;
-                    const int s = e >> 3, j = e & 7;
-                    K[s][j] = (bf16_t)(kf[e] * up);
-                    B[s][j] = (bf16_t)(bf_[e] * up);
-                    Qp[s][j] = V6 ? (bf16_t)(xe >= base ? rf[e] * ex2(base - xe) : 0.f)
-                                  : (bf16_t)(xi >= base ? rf[e] * ex2(base - xi) : 0.f);
-                    Ap[s][j] = (bf16_t)(xe >= base ? af[e] * ex2(base - xe) : 0.f);
-                }
-#pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    *reinterpret_cast<bf16x8_t*>(smem + OFF_KT + ((w * 2 + s) * 64 + lane) * 16) = K[s];
-                    *reinterpret_cast<bf16x8_t*>(smem + OFF_BT + ((w * 2 + s) * 64 + lane) * 16) = B[s];
-                }
-                __syncthreads();
             }
+        };
+        // block (I, J) -> the sigma fragments of the [i][j] matrices / the row-major blocks of Aab
+        auto store_block = [&](const Set& a, int I, int J) {
+            const int off = ((fidx(I, J >> 1) * 64 + lane) * 8 + 4 * (J & 1)) * 2;
+            *reinterpret_cast<bf16x4_t*>(smem + OFF_AQK + off) = pack4(a.qk);
+            *reinterpret_cast<bf16x4_t*>(smem + OFF_AQB + off) = pack4(a.qb);
+            *reinterpret_cast<bf16x4_t*>(smem + OFF_AAK + off) = pack4(a.ak);
+            // row-major [i][j]: lane holds i = x, j = 4g..4g+3
+            if (J < I) *reinterpret_cast<bf16x4_t*>(smem + OFF_AAB + lidx(I, J) * 512 + (x * 16 + 4 * g) * 2) = pack4(a.ab);
+        };
+        Set D, S, F0, F1;
+        clear(D); clear(S); clear(F0); clear(F1);
+        const int n_other = w == 0 ? 2 : (w == 1 ? 1 : 0);     // blocks of another row
+        const int I_other = w == 0 ? 3 : 2;
+        block(D, w, QG, AG);
+#pragma unroll
+        for (int s = 0; s < 2; ++s)             // the diagonal block once more with the operands swapped: rows i, column j
+            if constexpr (!V6) diagX = mfma_bf16(AG[s], lds_read_frag(smem, OFF_BT, w * 2 + s, lane), diagX);
+        if (w >= 1) block(S, w - 1, QG, AG);
+        if (n_other >= 1) {
+            bf16x8_t Qo[2], Ao[2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                const int at = tile_at(16 * I_other + x, 32 * s + 8 * g);
+                Qo[s] = *reinterpret_cast<const bf16x8_t*>(smem + OFF_QG_P2 + at);
+                Ao[s] = *reinterpret_cast<const bf16x8_t*>(smem + OFF_AG + at);
+            }
+            block(F0, 0, Qo, Ao);
+            if (n_other == 2) block(F1, 1, Qo, Ao);
         }
+        // causal masks on the diagonal block: j <= i for Aqk/Aqb, j < i for Aak/Aab (j = 4g+e, i = x)
 #pragma unroll
-        for (int J = 0; J < 4; ++J) {
-            if (J <= w) {
-#pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    const bf16x8_t kt = lds_read_frag(smem, OFF_KT, J * 2 + s, lane);
-                    const bf16x8_t bt = lds_read_frag(smem, OFF_BT, J * 2 + s, lane);
-                    acc_qk[J] = mfma_bf16(kt, Qp[s], acc_qk[J]);
-                    if constexpr (!V6) {       // RWKV6: a = b = 0, these three stay zero
-                        acc_qb[J] = mfma_bf16(bt, Qp[s], acc_qb[J]);
-                        acc_ak[J] = mfma_bf16(kt, Ap[s], acc_ak[J]);
-                        acc_ab[J] = mfma_bf16(bt, Ap[s], acc_ab[J]);
+        for (int e = 0; e < 4; ++e) {
+            const int jj = 4 * g + e;
+            if (jj > x) { D.qk[e] = 0.f; D.qb[e] = 0.f; }
+            if constexpr (V6) { if (jj == x) D.qk[e] = bonus; }
+            if (jj >= x) { D.ak[e] = 0.f; D.ab[e] = 0.f; }
+            if (x >= jj) diagX[e] = 0.f;          // here rows are i = 4g+e, column j = x: keep j < i
+        }
+        diagXT = D.ab;
+        __syncthreads();                                                       // Bx: every wave has taken its V, and the copy of qg is done with
+        store_block(D, w, w);
+        if (w >= 1) store_block(S, w, w - 1);
+        if (n_other >= 1) store_block(F0, I_other, 0);
+        if (n_other == 2) store_block(F1, I_other, 1);
+    } else {
+        float4_t acc_qk[4], acc_qb[4], acc_ak[4], acc_ab[4];
+    #pragma unroll
+        for (int J = 0; J < 4; ++J) {           // tiles right of the diagonal block (J > w) are never touched
+            if (J <= w) { acc_qk[J] = zero4; acc_qb[J] = zero4; acc_ak[J] = zero4; acc_ab[J] = zero4; }
+        }
+        bf16x8_t Qp[2] = {QG[0], QG[1]}, Ap[2] = {AG[0], AG[1]};
+        for (int p = 0; p < np; ++p) {
+            if constexpr (!SINGLE) {
+                if (p > 0) {                    // rare: tokens whose cumulative decay lies in bucket p
+                    __syncthreads();
+                    const float base = BUCKET * (float)p;
+                    float xs2[16], X2[16];
+                    bf16x8_t W2[2], R2[2], K2[2], A2[2], B2[2];
+                    int lane_o = lane;
+                    asm volatile("" : "+v"(lane_o));
+                    const int64_t at = first_piece(lane_o);
+                    load2(w_, at, W2); load2(r_, at, R2); load2(k_, at, K2);
+                    if constexpr (V6) {
+                        A2[0] = A2[1] = B2[0] = B2[1] = load_frag_global(nullptr, false);
+                    } else {
+                        load2(a_, at, A2); load2(b_, at, B2);
+                    }
+                    if (ragged) {
+                        asm volatile("" ::: "memory");
+                        if (!valid) R2[0] = R2[1] = K2[0] = K2[1] = A2[0] = A2[1] = B2[0] = B2[1] = load_frag_global(nullptr, false);
+                    }
+                    decays(W2, xs2, X2);
+                    add_prefix(X2);
+                    float rf[16], kf[16], af[16], bf_[16];
+                    unpack8(R2[0], rf); unpack8(R2[1], rf + 8); unpack8(K2[0], kf); unpack8(K2[1], kf + 8);
+                    unpack8(A2[0], af); unpack8(A2[1], af + 8); unpack8(B2[0], bf_); unpack8(B2[1], bf_ + 8);
+    #pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const float xi = X2[e], xe = xi - xs2[e];        // xe: up to, not including, this token
+                        const float up = (xi >= base && xi < base + BUCKET) ? ex2(xi - base) : 0.f;
+                        const int s = e >> 3, j = e & 7;
+                        K[s][j] = (bf16_t)(kf[e] * up);
+                        B[s][j] = (bf16_t)(bf_[e] * up);
+                        Qp[s][j] = V6 ? (bf16_t)(xe >= base ? rf[e] * ex2(base - xe) : 0.f)
+                                      : (bf16_t)(xi >= base ? rf[e] * ex2(base - xi) : 0.f);
+                        Ap[s][j] = (bf16_t)(xe >= base ? af[e] * ex2(base - xe) : 0.f);
+                    }
+    #pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        *reinterpret_cast<bf16x8_t*>(smem + OFF_KT + ((w * 2 + s) * 64 + lane) * 16) = K[s];
+                        *reinterpret_cast<bf16x8_t*>(smem + OFF_BT + ((w * 2 + s) * 64 + lane) * 16) = B[s];
+                    }
+                    __syncthreads();
+                }
+            }
+    #pragma unroll
+            for (int J = 0; J < 4; ++J) {
+                if (J <= w) {
+    #pragma unroll
+                    for (int s = 0; s < 2; ++s) {
+                        const bf16x8_t kt = lds_read_frag(smem, OFF_KT, J * 2 + s, lane);
+                        const bf16x8_t bt = lds_read_frag(smem, OFF_BT, J * 2 + s, lane);
+                        acc_qk[J] = mfma_bf16(kt, Qp[s], acc_qk[J]);
+                        if constexpr (!V6) {       // RWKV6: a = b = 0, these three stay zero
+                            acc_qb[J] = mfma_bf16(bt, Qp[s], acc_qb[J]);
+                            acc_ak[J] = mfma_bf16(kt, Ap[s], acc_ak[J]);
+                            acc_ab[J] = mfma_bf16(bt, Ap[s], acc_ab[J]);
+                        }
                     }
                 }
             }
+            // the diagonal block once more with the operands swapped: rows i, column j
+    #pragma unroll
+            for (int s = 0; s < 2; ++s)
+                if constexpr (!V6) diagX = mfma_bf16(Ap[s], lds_read_frag(smem, OFF_BT, w * 2 + s, lane), diagX);
         }
-        // the diagonal block once more with the operands swapped: rows i, column j
-#pragma unroll
-        for (int s = 0; s < 2; ++s)
-            if constexpr (!V6) diagX = mfma_bf16(Ap[s], lds_read_frag(smem, OFF_BT, w * 2 + s, lane), diagX);
-    }
-    float4_t diagXT = zero4;                // D layout of X^T (rows j, column i)
-    // causal masks on the diagonal block: j <= i for Aqk/Aqb, j < i for Aak/Aab (j = 4g+e, i = x)
-#pragma unroll
-    for (int J = 0; J < 4; ++J) {
-        if (J == w) {
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int jj = 4 * g + e;
-                if (jj > x) { acc_qk[J][e] = 0.f; acc_qb[J][e] = 0.f; }
-                if constexpr (V6) { if (jj == x) acc_qk[J][e] = bonus; }
-                if (jj >= x) { acc_ak[J][e] = 0.f; acc_ab[J][e] = 0.f; }
-                if (x >= jj) diagX[e] = 0.f;          // here rows are i = 4g+e, column j = x: keep j < i
+        // causal masks on the diagonal block: j <= i for Aqk/Aqb, j < i for Aak/Aab (j = 4g+e, i = x)
+    #pragma unroll
+        for (int J = 0; J < 4; ++J) {
+            if (J == w) {
+    #pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int jj = 4 * g + e;
+                    if (jj > x) { acc_qk[J][e] = 0.f; acc_qb[J][e] = 0.f; }
+                    if constexpr (V6) { if (jj == x) acc_qk[J][e] = bonus; }
+                    if (jj >= x) { acc_ak[J][e] = 0.f; acc_ab[J][e] = 0.f; }
+                    if (x >= jj) diagX[e] = 0.f;          // here rows are i = 4g+e, column j = x: keep j < i
+                }
+                diagXT = acc_ab[J];
             }
-            diagXT = acc_ab[J];
         }
-    }
-    __syncthreads();                                                           // Bx: every wave has taken its V
-#pragma unroll
-    for (int J = 0; J < 4; ++J) {
-        if (J <= w) {
-            const int f = fidx(w, J >> 1);
-            const int off = ((f * 64 + lane) * 8 + 4 * (J & 1)) * 2;
-            *reinterpret_cast<bf16x4_t*>(smem + OFF_AQK + off) = pack4(acc_qk[J]);
-            *reinterpret_cast<bf16x4_t*>(smem + OFF_AQB + off) = pack4(acc_qb[J]);
-            *reinterpret_cast<bf16x4_t*>(smem + OFF_AAK + off) = pack4(acc_ak[J]);
-            if (J < w) {
-                // block (w, J), row-major [i][j]: lane holds i = x, j = 4g..4g+3
-                *reinterpret_cast<bf16x4_t*>(smem + OFF_AAB + lidx(w, J) * 512 + (x * 16 + 4 * g) * 2) = pack4(acc_ab[J]);
+        __syncthreads();                                                           // Bx: every wave has taken its V
+    #pragma unroll
+        for (int J = 0; J < 4; ++J) {
+            if (J <= w) {
+                const int f = fidx(w, J >> 1);
+                const int off = ((f * 64 + lane) * 8 + 4 * (J & 1)) * 2;
+                *reinterpret_cast<bf16x4_t*>(smem + OFF_AQK + off) = pack4(acc_qk[J]);
+                *reinterpret_cast<bf16x4_t*>(smem + OFF_AQB + off) = pack4(acc_qb[J]);
+                *reinterpret_cast<bf16x4_t*>(smem + OFF_AAK + off) = pack4(acc_ak[J]);
+                if (J < w) {
+                    // block (w, J), row-major [i][j]: lane holds i = x, j = 4g..4g+3
+                    *reinterpret_cast<bf16x4_t*>(smem + OFF_AAB + lidx(w, J) * 512 + (x * 16 + 4 * g) * 2) = pack4(acc_ab[J]);
+                }
             }
         }
     }
