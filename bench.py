@@ -43,7 +43,7 @@ N = 64
 # `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` on this same command, each scaled by what the
 # counter reads for a plain 1 GiB copy (FETCH_SIZE x2.000, WRITE_SIZE x1.000); the summary is
 # profiles/fwd_chunk_prefill_and_decode_traffic.txt.
-MEASURED_TRAFFIC_BYTES = 1537714894
+MEASURED_TRAFFIC_BYTES = 1536130562
 TRAFFIC_SOURCE = ("profiles/fwd_chunk_prefill_and_decode_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this "
                   "command at B=8 T=4096 H=32; a constant, not measured in this run)")
 EXEC_FLOPS_SOURCE = ("profiles/fwd_chunk_prefill_mfma_counters.txt (SQ_INSTS_VALU_MFMA_MOPS_BF16: 118,784 flop per "
@@ -54,7 +54,7 @@ EXEC_FLOPS_SOURCE = ("profiles/fwd_chunk_prefill_mfma_counters.txt (SQ_INSTS_VAL
 # kernel sources (sources_digest() below) at that time.  The JSON line carries this digest next to the digest of
 # the sources in the tree and of the loaded library, so a reader sees whether the constants still belong to
 # the code that was timed.
-CONSTANTS_SOURCES_DIGEST = "12d15a0fc730c853"
+CONSTANTS_SOURCES_DIGEST = "55ac6daa92b2ca87"
 
 
 def sources_digest():
