@@ -18,6 +18,7 @@ __version__ = "0.1"
 
 from .rwkv7 import generalized_delta_rule as _hip_generalized_delta_rule
 from .rwkv7 import rwkv7_decode_step, last_forward_status  # noqa: F401
+from .rwkv7 import generalized_delta_rule_resets  # noqa: F401
 from .rwkv6 import get_rwkv6_kernel
 
 
