@@ -21,12 +21,13 @@ def run_both(xs, device, **kw):
     return o, s, o_ref, s_ref
 
 
-# B*H < 96 takes the two-kernel form (summaries in HBM, then the scan), B*H >= 96 the one-kernel
-# form with the state handed from chunk to chunk: both are covered
+# B*H < 72 takes the two-kernel form (summaries in HBM, then the scan), B*H >= 72 the one-kernel
+# form with the state handed from chunk to chunk: both are covered, and both sides of the threshold
 @pytest.mark.parametrize("B,T,H", [(1, 64, 1), (1, 128, 2), (2, 256, 4), (1, 100, 3), (2, 37, 2),
                                    (1, 2, 1), (3, 65, 5), (1, 1024, 2),
                                    (4, 200, 32), (8, 64, 16), (2, 130, 64), (16, 3, 8), (5, 577, 40), (3, 130, 32),
                                    (4, 130, 25), (1, 200, 97),            # fused, B*H not a multiple of 8 (hand-off across XCDs)
+                                   (1, 330, 71), (1, 330, 72),            # the last two-kernel and the first one-kernel head count
                                    (2, 8192, 48)])                        # fused, 128 chunks per sequence
 def test_chunked_matches_oracle(device, B, T, H):
     xs = make_inputs(B, T, H, 64, seed=1000 + T, dtype=torch.bfloat16)
