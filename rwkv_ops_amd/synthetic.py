@@ -38,10 +38,11 @@ def make_inputs(B, T, H, N=64, *, seed=0, dtype=torch.float32, h0=True, h0_batch
 
 # Relative-L2 thresholds of the bf16 backward against float32 autograd through the oracle on the same rounded
 # inputs, per gradient (the reference states none).  Largest values measured over the GPU tests: dr 3.3e-3,
-# dw 3.5e-3, dk 3.7e-3, dv 3.7e-3, dh0 3.2e-3; da 5.4e-3 and db 5.9e-3 (short sequences; 4.7e-3 at the training
-# shape): these two pass through the triangular inverse and its adjoint, two more bf16 roundings than the others.
+# dw 3.5e-3, dk 3.7e-3, dv 3.7e-3, dh0 3.2e-3; da 5.4e-3 and db 5.9e-3 (the latter on a single 64-token chunk of one
+# head, 5.1e-3 otherwise; 4.7e-3 at the training shape): these two pass through the triangular inverse and its
+# adjoint, two more bf16 roundings than the others.
 GRAD_NAMES = ("dr", "dw", "dk", "dv", "da", "db", "dh0")
-GRAD_TOL = {"dr": 5e-3, "dw": 5e-3, "dk": 5e-3, "dv": 5e-3, "da": 7e-3, "db": 7e-3, "dh0": 5e-3}
+GRAD_TOL = {"dr": 5e-3, "dw": 5e-3, "dk": 5e-3, "dv": 5e-3, "da": 6e-3, "db": 6e-3, "dh0": 5e-3}
 
 
 def rel_l2(x, ref):
